@@ -1,0 +1,168 @@
+/*
+ * tritonformer_amd.h — C ABI of libtritonformer_amd.so (gfx950 / MI355X).
+ *
+ * The reference (fattorib/tritonformer) has no FFI: its boundary is a set of
+ * Python launcher functions under tritonformer/kernels/ that take torch tensors
+ * and start Triton kernels on the current stream.  Each entry point below
+ * replaces one (or a fused group) of those launchers and is what a ctypes
+ * binding on the reference side would call.
+ *
+ * Conventions
+ *  - every pointer is a DEVICE pointer unless said otherwise; the library
+ *    never allocates, frees, retains or synchronises; work is enqueued on
+ *    `stream` (a hipStream_t passed as void*, NULL = the null stream);
+ *  - strides and leading dimensions are in ELEMENTS, sizes in elements;
+ *  - `dtype`: TF_F16 / TF_BF16 for the 16-bit paths, TF_F32 only where stated;
+ *  - return value: TF_OK (0) or a negative TF_E* code; tf_status_string()
+ *    gives the text.  Argument checks run on the host before any launch, so a
+ *    non-zero status means nothing was enqueued.
+ */
+#ifndef TRITONFORMER_AMD_H
+#define TRITONFORMER_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum tf_dtype { TF_F16 = 0, TF_BF16 = 1, TF_F32 = 2 };
+
+enum tf_status {
+  TF_OK = 0,
+  TF_EINVAL = -1,    /* bad size / null pointer / unsupported combination   */
+  TF_EDTYPE = -2,    /* dtype not supported by this entry point             */
+  TF_EALIGN = -3,    /* pointer or stride violates a stated alignment rule  */
+  TF_ESHAPE = -4,    /* shape precondition of the reference violated        */
+  TF_EWORKSPACE = -5,/* workspace missing or too small                      */
+  TF_ELAUNCH = -6    /* the HIP runtime refused the launch                  */
+};
+
+/* Operand storage for tf_gemm.  "K" is the contraction dimension.
+ *   TF_OP_KMAJOR : element (row, k) at  ptr[row * ld + k]   (k contiguous)
+ *   TF_OP_KMINOR : element (row, k) at  ptr[k * ld + row]   (row contiguous)
+ * where "row" is m for A and n for B. */
+enum tf_op_layout { TF_OP_KMAJOR = 0, TF_OP_KMINOR = 1 };
+
+const char* tf_status_string(int status);
+int tf_version(void);
+
+/* ---- dense contractions (fp16/bf16 MFMA, fp32 accumulate) --------------- */
+
+/* C[M,N] = epilogue( sum_k A(m,k) * B(n,k) ),  epilogue = (+bias[n]) then
+ * optional max(.,0), rounded once to `dtype`.
+ * Replaces mm / gemm / bmm (+ the torch.sum over the batch that follows bmm):
+ *   tritonformer/kernels/gemm.py:361-401 (mm, optional ReLU)
+ *   tritonformer/kernels/gemm.py:572-616 (gemm: bias, optional ReLU)
+ *   tritonformer/kernels/gemm.py:161-200 (bmm) + tritonformer/linear.py:24-25
+ * Forward      Y = X W      : A = X  KMAJOR (M=B*S, K=in),  B = W  KMINOR.
+ * Input grad   dX = dY W^T  : A = dY KMAJOR (K=out),        B = W  KMAJOR.
+ * Weight grad  dW = X^T dY  : A = X  KMINOR (M=in, K=B*S),  B = dY KMINOR;
+ *   the batch dimension is part of the contraction, so no (B,in,out)
+ *   temporary exists.
+ * `workspace` (fp32, tf_gemm_workspace_bytes() bytes) is needed only when that
+ * query returns non-zero (contraction split over several workgroups, summed in
+ * a fixed order by a second kernel: results are bitwise reproducible).
+ * Fast path needs 16-byte aligned pointers and contiguous-dimension extents
+ * and leading dimensions that are multiples of 8; anything else takes a
+ * slower element-wise-load path with identical arithmetic. */
+int tf_gemm(void* stream, int dtype, int layout_a, int layout_b,
+            int64_t M, int64_t N, int64_t K,
+            const void* A, int64_t lda, const void* B, int64_t ldb,
+            void* C, int64_t ldc, const void* bias, int relu,
+            void* workspace, int64_t workspace_bytes);
+int64_t tf_gemm_workspace_bytes(int layout_a, int layout_b, int64_t M, int64_t N, int64_t K);
+
+/* Causal flash attention forward.  q,k,v,o: logical (B, nh, S, hd) with the
+ * SAME element strides {sb, sh, ss} and unit stride along hd (the reference
+ * passes q's strides for all four, kernels/attention.py:202-205).
+ * lse: (B, nh, S) fp32, contiguous, log2-domain log-sum-exp of the scaled
+ * (and biased) scores.  bias: NULL, or (nh, Sb, Sb) with Sb >= S, element
+ * strides {bias_sh, bias_sr}, unit stride along keys, added after scaling
+ * (kernels/biased_attention.py:101-106); -inf entries are allowed.
+ * Replaces flash_wrapper_fwd (kernels/attention.py:171-217) and
+ * flash_wrapper_fwd_attn_bias (kernels/biased_attention.py:188-245).
+ * Preconditions (as the reference asserts): hd in {32,64,128}; S % 64 == 0. */
+int tf_attn_fwd(void* stream, int dtype, int64_t B, int64_t nh, int64_t S, int64_t hd,
+                const void* q, const void* k, const void* v, void* o,
+                int64_t sb, int64_t sh, int64_t ss,
+                float* lse, const void* bias, int64_t bias_sh, int64_t bias_sr,
+                float scale);
+
+/* Backward of the above: dq, dk, dv have q's strides.  delta: (B, nh, S) fp32
+ * scratch (row sums of dO*O), written then read by this call.
+ * Replaces flash_wrapper_bwd (kernels/attention.py:550-607) and
+ * flash_wrapper_bwd_attn_bias (kernels/biased_attention.py:598-660).
+ * No gradient is produced for the bias (tritonformer/attention.py:60). */
+int tf_attn_bwd(void* stream, int dtype, int64_t B, int64_t nh, int64_t S, int64_t hd,
+                const void* q, const void* k, const void* v, const void* o, const void* d_o,
+                void* dq, void* dk, void* dv,
+                int64_t sb, int64_t sh, int64_t ss,
+                const float* lse, float* delta,
+                const void* bias, int64_t bias_sh, int64_t bias_sr, float scale);
+
+/* ---- bandwidth-bound kernels -------------------------------------------- */
+
+/* y = gamma * (x - mean) * rstd + beta over the last dimension; biased
+ * variance, rstd = 1/sqrt(var + eps), statistics in fp32
+ * (kernels/layernorm.py:8-61, launcher :64-87).  mean/rstd: (rows) fp32, saved
+ * for the backward pass (the reference recomputes them instead). */
+int tf_layernorm_fwd(void* stream, int dtype, int64_t rows, int64_t d,
+                     const void* x, int64_t ldx, const void* gamma, const void* beta,
+                     float eps, void* y, int64_t ldy, float* mean, float* rstd);
+
+/* dx, dgamma, dbeta in one pass over (dy, x) plus a small second-stage
+ * reduction.  Replaces dx_layernorm (kernels/layernorm.py:140-162) and
+ * layernorm_da_db (kernels/layernorm.py:226-259, with its reductions.py
+ * second stage).  partial: fp32 scratch of tf_layernorm_bwd_partial_bytes(). */
+int tf_layernorm_bwd(void* stream, int dtype, int64_t rows, int64_t d,
+                     const void* dy, int64_t lddy, const void* x, int64_t ldx,
+                     const void* gamma, const float* mean, const float* rstd,
+                     void* dx, int64_t lddx, void* dgamma, void* dbeta,
+                     float* partial, int64_t partial_bytes);
+int64_t tf_layernorm_bwd_partial_bytes(int64_t rows, int64_t d);
+
+/* Row softmax / its backward dx = y * (dy - sum(y*dy)); dtype f16/bf16/f32.
+ * Replaces softmax_fwd / softmax_bwd (kernels/softmax.py:37-54, 95-111); the
+ * backward writes a new buffer instead of overwriting grad_out. */
+int tf_softmax_fwd(void* stream, int dtype, int64_t rows, int64_t cols,
+                   const void* x, int64_t ldx, void* y, int64_t ldy);
+int tf_softmax_bwd(void* stream, int dtype, int64_t rows, int64_t cols,
+                   const void* dy, int64_t lddy, const void* y, int64_t ldy,
+                   void* dx, int64_t lddx);
+
+/* Per-row loss[r] = logsumexp(logits[r,:]) - logits[r, labels[r]] with an
+ * online max/sum single pass; also stores lse[r] (natural log, fp32).
+ * labels: int64, each in [0, V).  loss has `dtype`.
+ * Replaces cross_entropy_fwd (kernels/crossentropy.py:47-75). */
+int tf_cross_entropy_fwd(void* stream, int dtype, int64_t rows, int64_t V,
+                         const void* logits, int64_t ld, const int64_t* labels,
+                         void* loss, float* lse);
+
+/* dlogits[r,v] = (exp(logits[r,v] - lse[r]) - [v == labels[r]]) * gout[r].
+ * Replaces cross_entropy_bwd (kernels/crossentropy.py:110-127) and the
+ * broadcast multiply in tritonformer/crossentropy.py:24.  gout has `dtype`;
+ * gout_stride 0 broadcasts one value. */
+int tf_cross_entropy_bwd(void* stream, int dtype, int64_t rows, int64_t V,
+                         const void* logits, int64_t ld, const int64_t* labels,
+                         const float* lse, const void* gout, int64_t gout_stride,
+                         void* dlogits, int64_t ldd);
+
+/* out[c] = sum_r x[r, c] with fp32 accumulation (bias gradient).
+ * Replaces unbroadcast_leading (kernels/reductions.py:97-122, two-stage with
+ * _unbroadcast :57-63).  partial: fp32 scratch of tf_colsum_partial_bytes(). */
+int tf_colsum(void* stream, int dtype, int64_t rows, int64_t cols,
+              const void* x, int64_t ldx, void* out,
+              float* partial, int64_t partial_bytes);
+int64_t tf_colsum_partial_bytes(int64_t rows, int64_t cols);
+
+/* out = where(act > 0, grad, 0), out of place.
+ * Replaces mask_grad (kernels/activation.py:27-44), which works in place. */
+int tf_relu_mask(void* stream, int dtype, int64_t rows, int64_t cols,
+                 const void* grad, int64_t ldg, const void* act, int64_t lda,
+                 void* out, int64_t ldo);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TRITONFORMER_AMD_H */

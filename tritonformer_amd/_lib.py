@@ -1,0 +1,91 @@
+"""ctypes binding of libtritonformer_amd.so (the C ABI in include/tritonformer_amd.h).
+
+The HIP library is the only execution path of this package: if it cannot be
+loaded the import of any operator raises, there is no PyTorch/CPU fallback.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libtritonformer_amd.so")
+
+TF_F16, TF_BF16, TF_F32 = 0, 1, 2
+KMAJOR, KMINOR = 0, 1
+
+_c = ctypes
+_vp, _i, _i64, _f = _c.c_void_p, _c.c_int, _c.c_int64, _c.c_float
+
+# name -> (restype, argtypes); mirrors include/tritonformer_amd.h one to one
+SIGNATURES = {
+    "tf_status_string": (_c.c_char_p, [_i]),
+    "tf_version": (_i, []),
+    "tf_gemm": (_i, [_vp, _i, _i, _i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i, _vp, _i64]),
+    "tf_gemm_workspace_bytes": (_i64, [_i, _i, _i64, _i64, _i64]),
+    "tf_attn_fwd": (_i, [_vp, _i, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _i64, _f]),
+    "tf_attn_bwd": (_i, [_vp, _i, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64,
+                         _vp, _vp, _vp, _i64, _i64, _f]),
+    "tf_layernorm_fwd": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _vp, _vp, _f, _vp, _i64, _vp, _vp]),
+    "tf_layernorm_bwd": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _i64]),
+    "tf_layernorm_bwd_partial_bytes": (_i64, [_i64, _i64]),
+    "tf_softmax_fwd": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _vp, _i64]),
+    "tf_softmax_bwd": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64]),
+    "tf_cross_entropy_fwd": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _vp, _vp, _vp]),
+    "tf_cross_entropy_bwd": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _vp, _i64]),
+    "tf_colsum": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _vp, _vp, _i64]),
+    "tf_colsum_partial_bytes": (_i64, [_i64, _i64]),
+    "tf_relu_mask": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64]),
+}
+
+_lib = None
+
+
+def load():
+    """Load the shared library once; raise if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} is missing: build it with `python -m tritonformer_amd._build` "
+                "(there is no fallback path)"
+            )
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+class TritonformerAmdError(RuntimeError):
+    pass
+
+
+def check(status):
+    if status != 0:
+        msg = load().tf_status_string(status).decode()
+        if status in (-1, -3, -4):
+            raise ValueError(f"tritonformer_amd: {msg}")
+        raise TritonformerAmdError(f"tritonformer_amd: {msg}")
+
+
+def dtype_code(t):
+    if t == torch.float16:
+        return TF_F16
+    if t == torch.bfloat16:
+        return TF_BF16
+    if t == torch.float32:
+        return TF_F32
+    raise TypeError(f"tritonformer_amd: unsupported dtype {t}")
+
+
+def stream_ptr():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def require_cuda(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise ValueError("tritonformer_amd kernels need tensors on the GPU (there is no CPU path)")

@@ -1,0 +1,671 @@
+// Causal flash attention forward / backward on gfx950 MFMA, optional additive
+// bias (ALiBi).  FlashAttention-2 schedule: the forward and the dQ pass are
+// partitioned over query blocks with a loop over key/value blocks up to the
+// diagonal; the dK/dV pass is partitioned over key/value blocks with a loop
+// over the query blocks at or below the diagonal.  No atomics: results are
+// bitwise reproducible.
+//
+// Layout trick used by all three kernels: score tiles are produced
+// TRANSPOSED with respect to the operand that stays in registers, i.e. the
+// 32x32 MFMA output has the register-resident index (query in the forward and
+// dQ passes, key in the dK/dV pass) along lanes.  Then
+//   * per-row softmax statistics are per-lane scalars (one cross-lane op to
+//     merge the two half-waves),
+//   * the fp32 tile, rounded to 16 bit, already IS the k-contiguous MFMA
+//     operand of the second contraction: no LDS round trip for P / dS,
+//   * the other operand of the second contraction (V, dO, Q or K, stored
+//     row-major [seq][hd] in LDS) is fetched with the transposing
+//     ds_read_b64_tr_b16.
+// The 16 contraction slots of lane-half h in step t map to sequence offsets
+// 16t + 8(s/4) + 4h + s%4 (s = 0..7), on both operands alike.
+#include "rowops.h"
+
+namespace tfa {
+
+struct AttnParams {
+  const void *q, *k, *v, *o, *d_o;
+  void *out, *dq, *dk, *dv;
+  float* lse;    // written by fwd, read by bwd
+  float* delta;  // written by the bwd pre-pass
+  const void* bias;
+  int64_t sb, sh, ss;         // element strides of q/k/v/o and their grads
+  int64_t bias_sh, bias_sr;   // element strides of bias (head, query row)
+  int B, nh, S;
+  float scale_log2;           // scale * log2(e)
+  float scale;
+};
+
+// ---------------------------------------------------------------------------
+// LDS tile [ROWS][HD] of 16-bit elements, hd contiguous, chunk-swizzled so that
+// both the row-wise 16-byte reads and the transposing 8-byte reads are free of
+// bank conflicts.
+// ---------------------------------------------------------------------------
+template <typename T, int ROWS, int HD>
+struct SeqTile {
+  static constexpr int CPR = HD / 8;
+  static constexpr int BYTES = ROWS * HD * 2;
+  static constexpr int PER_THREAD = (ROWS * CPR + 255) / 256;
+  typedef typename Vec<T>::v8 v8;
+
+  static __device__ __forceinline__ int swz(int row) {
+    if (CPR == 4) return (row >> 2) & 3;
+    if (CPR == 8) { const int u = (row >> 1) & 7; return ((u & 1) << 2) | (u >> 1); }
+    return ((row & 3) << 2) | ((row >> 2) & 3);
+  }
+  static __device__ __forceinline__ int addr(int row, int chunk) { return (row * CPR + (chunk ^ swz(row))) * 16; }
+
+  // rows [row0, row0+ROWS) of a (seq, hd) matrix with row stride ss; always in bounds.
+  static __device__ __forceinline__ void fetch(u32x4 (&regs)[PER_THREAD], const T* __restrict__ base, int64_t ss,
+                                               int row0) {
+#pragma unroll
+    for (int j = 0; j < PER_THREAD; ++j) {
+      const int id = threadIdx.x + j * 256;
+      if (ROWS * CPR % 256 == 0 || id < ROWS * CPR) {
+        const int row = id / CPR, c = id % CPR;
+        regs[j] = ld16(base + (int64_t)(row0 + row) * ss + c * 8);
+      }
+    }
+  }
+  static __device__ __forceinline__ void commit(char* lds, const u32x4 (&regs)[PER_THREAD]) {
+#pragma unroll
+    for (int j = 0; j < PER_THREAD; ++j) {
+      const int id = threadIdx.x + j * 256;
+      if (ROWS * CPR % 256 == 0 || id < ROWS * CPR) lds_st16(lds, addr(id / CPR, id % CPR), regs[j]);
+    }
+  }
+  // Operand with the tile's rows as the MFMA row/col index: lane l gets
+  // (row rb + l%32, hd = ks*16 + (l/32)*8 + 0..7).
+  static __device__ __forceinline__ v8 frag_rows(const char* lds, int rb, int ks, int lane) {
+    return __builtin_bit_cast(v8, lds_ld16(lds, addr(rb + (lane & 31), ks * 2 + (lane >> 5))));
+  }
+  // Operand with hd as the MFMA row/col index and the tile's rows as the
+  // contraction: lane l gets (hd = dt*32 + l%32, rows rb16 + 8*(s/4) + 4*(l/32) + s%4).
+  static __device__ __forceinline__ v8 frag_hd(const char* lds, int rb16, int dt, int lane) {
+    const int i = lane & 15;
+    const int col = dt * 32 + 16 * ((lane >> 4) & 1) + (i & 3) * 4;
+    const int r0 = rb16 + 4 * (lane >> 5) + (i >> 2);
+    const u32x2 lo = lds_ld8_tr(lds, addr(r0, col >> 3) + (col & 7) * 2);
+    const u32x2 hi = lds_ld8_tr(lds, addr(r0 + 8, col >> 3) + (col & 7) * 2);
+    u32x4 v = {lo[0], lo[1], hi[0], hi[1]};
+    return __builtin_bit_cast(v8, v);
+  }
+};
+
+template <typename T> __device__ __forceinline__ typename Vec<T>::v8 round8(const f32x16& x, int t) {
+  typename Vec<T>::v8 r;
+#pragma unroll
+  for (int s = 0; s < 8; ++s) r[s] = (T)x[t * 8 + s];
+  return r;
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Register r of a 32x32 MFMA result covers row (r/4)*8 + 4*(lane/32) + r%4.
+__device__ __forceinline__ int reg_row(int r, int lane) { return (r >> 2) * 8 + 4 * (lane >> 5) + (r & 3); }
+
+// ===========================================================================
+// Forward.  Workgroup: 4 waves x 32 queries; key/value blocks of 64.
+// ===========================================================================
+template <typename T, int HD, bool HAS_BIAS>
+__global__ __launch_bounds__(256) void attn_fwd_kernel(AttnParams p) {
+  typedef SeqTile<T, 64, HD> KT;
+  typedef typename Vec<T>::v8 v8;
+  typedef typename Vec<T>::v4 v4;
+  constexpr int KS = HD / 16, DT = HD / 32;
+  constexpr int STAGE = 2 * KT::BYTES;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nbh = p.B * p.nh;
+  const int nqb = (p.S + 127) / 128;
+  const int qblk = nqb - 1 - (int)(blockIdx.x / nbh);  // heaviest query blocks first
+  const int bh = blockIdx.x % nbh;
+  const int b = bh / p.nh, h = bh % p.nh;
+  const int64_t base = (int64_t)b * p.sb + (int64_t)h * p.sh;
+  const T* Q = (const T*)p.q + base;
+  const T* K = (const T*)p.k + base;
+  const T* V = (const T*)p.v + base;
+  T* O = (T*)p.out + base;
+
+  const int q0 = qblk * 128;
+  const int q0w = q0 + wave * 32;
+  const bool active = q0w < p.S;
+  const int myq = q0w + (lane & 31);
+  const int kv_end = min(p.S, q0 + 128);
+  const int nkv = kv_end / 64;
+
+  v8 qf[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    u32x4 raw = {0u, 0u, 0u, 0u};
+    if (active) raw = ld16(Q + (int64_t)myq * p.ss + ks * 16 + (lane >> 5) * 8);
+    qf[ks] = __builtin_bit_cast(v8, raw);
+  }
+
+  f32x16 oacc[DT];
+#pragma unroll
+  for (int d = 0; d < DT; ++d)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) oacc[d][r] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+
+  u32x4 rk[KT::PER_THREAD], rv[KT::PER_THREAD];
+  KT::fetch(rk, K, p.ss, 0);
+  KT::fetch(rv, V, p.ss, 0);
+  KT::commit(smem, rk);
+  KT::commit(smem + KT::BYTES, rv);
+  __syncthreads();
+
+  for (int j = 0; j < nkv; ++j) {
+    const char* sk = smem + (j & 1) * STAGE;
+    const char* sv = sk + KT::BYTES;
+    const bool more = j + 1 < nkv;
+    if (more) {
+      KT::fetch(rk, K, p.ss, (j + 1) * 64);
+      KT::fetch(rv, V, p.ss, (j + 1) * 64);
+    }
+    const int kb = j * 64;
+    if (active && kb <= q0w + 31) {
+      const bool live1 = kb + 32 <= q0w + 31;  // second 32-key half not fully above the diagonal
+      f32x16 st[2];
+#pragma unroll
+      for (int jt = 0; jt < 2; ++jt) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) st[jt][r] = 0.f;
+        if (jt == 0 || live1) {
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) st[jt] = mfma32(KT::frag_rows(sk, jt * 32, ks, lane), qf[ks], st[jt]);
+        }
+      }
+      // scale, bias, causal mask; running max
+      float mx = -INFINITY;
+#pragma unroll
+      for (int jt = 0; jt < 2; ++jt) {
+        const bool live = jt == 0 || live1;
+        const bool diag = kb + jt * 32 + 31 > q0w;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int key0 = kb + jt * 32 + g * 8 + 4 * (lane >> 5);
+          float bv[4] = {0.f, 0.f, 0.f, 0.f};
+          if (HAS_BIAS && live) {
+            const v4 raw = *reinterpret_cast<const v4*>((const T*)p.bias + (int64_t)h * p.bias_sh +
+                                                        (int64_t)myq * p.bias_sr + key0);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) bv[e] = (float)raw[e] * kLog2e;
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            float s = st[jt][g * 4 + e] * p.scale_log2 + bv[e];
+            if (!live || (diag && key0 + e > myq)) s = -INFINITY;
+            st[jt][g * 4 + e] = s;
+            mx = fmaxf(mx, s);
+          }
+        }
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m_run, mx);
+      const float m_use = m_new == -INFINITY ? 0.f : m_new;
+      const float alpha = fast_exp2(m_run - m_use);
+      m_run = m_new;
+      float rs = 0.f;
+#pragma unroll
+      for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float e = fast_exp2(st[jt][r] - m_use);
+          st[jt][r] = e;
+          rs += e;
+        }
+      l_run = l_run * alpha + rs;
+#pragma unroll
+      for (int d = 0; d < DT; ++d)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[d][r] *= alpha;
+#pragma unroll
+      for (int jt = 0; jt < 2; ++jt) {
+        if (jt == 0 || live1) {
+#pragma unroll
+          for (int t = 0; t < 2; ++t) {
+            const v8 pb = round8<T>(st[jt], t);
+#pragma unroll
+            for (int d = 0; d < DT; ++d) oacc[d] = mfma32(KT::frag_hd(sv, jt * 32 + t * 16, d, lane), pb, oacc[d]);
+          }
+        }
+      }
+    }
+    if (more) {
+      char* dk = smem + ((j + 1) & 1) * STAGE;
+      KT::commit(dk, rk);
+      KT::commit(dk + KT::BYTES, rv);
+    }
+    __syncthreads();
+  }
+
+  if (active) {
+    const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+    const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+    if (lane < 32) p.lse[(int64_t)bh * p.S + myq] = m_run + log2f(l_tot);
+#pragma unroll
+    for (int d = 0; d < DT; ++d)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        v4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = (T)(oacc[d][g * 4 + e] * inv);
+        *reinterpret_cast<v4*>(O + (int64_t)myq * p.ss + d * 32 + g * 8 + 4 * (lane >> 5)) = o;
+      }
+  }
+}
+
+// ===========================================================================
+// Backward pre-pass: delta[b,h,q] = sum_d dO[q,d] * O[q,d].
+// ===========================================================================
+template <typename T, int HD>
+__global__ __launch_bounds__(256) void attn_delta_kernel(AttnParams p) {
+  constexpr int LPR = HD / 8;       // lanes per row
+  constexpr int RPB = 256 / LPR;    // rows per workgroup
+  const int nbh = p.B * p.nh;
+  const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / LPR;  // over nbh * S
+  if (row >= (int64_t)nbh * p.S) return;
+  const int bh = (int)(row / p.S), s = (int)(row % p.S);
+  const int64_t off = (int64_t)(bh / p.nh) * p.sb + (int64_t)(bh % p.nh) * p.sh + (int64_t)s * p.ss +
+                      (threadIdx.x % LPR) * 8;
+  float a[8], g[8];
+  Chunk<T>::load((const T*)p.o + off, a);
+  Chunk<T>::load((const T*)p.d_o + off, g);
+  float acc = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc += a[e] * g[e];
+#pragma unroll
+  for (int o = LPR / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+  if (threadIdx.x % LPR == 0) p.delta[row] = acc;
+}
+
+// ===========================================================================
+// dK/dV pass.  Workgroup: 4 waves x 32 keys; query blocks of 64 from the
+// diagonal downwards.  Q and dO tiles (+ their lse / delta) go through LDS.
+// ===========================================================================
+template <typename T, int HD, bool HAS_BIAS>
+__global__ __launch_bounds__(256) void attn_dkdv_kernel(AttnParams p) {
+  typedef SeqTile<T, 64, HD> QT;
+  typedef typename Vec<T>::v8 v8;
+  typedef typename Vec<T>::v4 v4;
+  constexpr int KS = HD / 16, DT = HD / 32;
+  constexpr int STAGE = 2 * QT::BYTES + 2 * 64 * 4;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nbh = p.B * p.nh;
+  const int kblk = (int)(blockIdx.x / nbh);  // lowest key blocks (longest loops) first
+  const int bh = blockIdx.x % nbh;
+  const int b = bh / p.nh, h = bh % p.nh;
+  const int64_t base = (int64_t)b * p.sb + (int64_t)h * p.sh;
+  const T* Q = (const T*)p.q + base;
+  const T* K = (const T*)p.k + base;
+  const T* V = (const T*)p.v + base;
+  const T* dO = (const T*)p.d_o + base;
+  const float* lse = p.lse + (int64_t)bh * p.S;
+  const float* delta = p.delta + (int64_t)bh * p.S;
+
+  const int k0 = kblk * 128;
+  const int kw0 = k0 + wave * 32;
+  const bool active = kw0 < p.S;
+  const int mykey = kw0 + (lane & 31);
+
+  v8 kf[KS], vf[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    u32x4 a = {0u, 0u, 0u, 0u}, c = {0u, 0u, 0u, 0u};
+    if (active) {
+      a = ld16(K + (int64_t)mykey * p.ss + ks * 16 + (lane >> 5) * 8);
+      c = ld16(V + (int64_t)mykey * p.ss + ks * 16 + (lane >> 5) * 8);
+    }
+    kf[ks] = __builtin_bit_cast(v8, a);
+    vf[ks] = __builtin_bit_cast(v8, c);
+  }
+  f32x16 dk[DT], dv[DT];
+#pragma unroll
+  for (int d = 0; d < DT; ++d)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { dk[d][r] = 0.f; dv[d][r] = 0.f; }
+
+  const int nq = (p.S - k0) / 64;  // query blocks k0, k0+64, ...
+  u32x4 rq[QT::PER_THREAD], rdo[QT::PER_THREAD];
+  float rstat = 0.f;  // threads 0..63: lse, 64..127: delta of the block's 64 queries
+
+  auto fetch = [&](int qb) {
+    QT::fetch(rq, Q, p.ss, qb);
+    QT::fetch(rdo, dO, p.ss, qb);
+    if (threadIdx.x < 64) rstat = lse[qb + threadIdx.x];
+    else if (threadIdx.x < 128) rstat = delta[qb + threadIdx.x - 64];
+  };
+  auto commit = [&](char* st) {
+    QT::commit(st, rq);
+    QT::commit(st + QT::BYTES, rdo);
+    if (threadIdx.x < 128) reinterpret_cast<float*>(st + 2 * QT::BYTES)[threadIdx.x] = rstat;
+  };
+
+  if (nq > 0) { fetch(k0); commit(smem); }
+  __syncthreads();
+
+  for (int it = 0; it < nq; ++it) {
+    const char* sq = smem + (it & 1) * STAGE;
+    const char* sdo = sq + QT::BYTES;
+    const float* sstat = reinterpret_cast<const float*>(sq + 2 * QT::BYTES);
+    const bool more = it + 1 < nq;
+    const int qb = k0 + it * 64;
+    if (more) fetch(qb + 64);
+    if (active) {
+#pragma unroll
+      for (int qt = 0; qt < 2; ++qt) {
+        const int qs = qb + qt * 32;      // first query of this 32-row sub-tile
+        if (qs + 31 < kw0) continue;      // entirely above the diagonal for this wave
+        const bool diag = qs < kw0 + 31;
+        f32x16 s, dp;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          s = mfma32(QT::frag_rows(sq, qt * 32, ks, lane), kf[ks], s);
+          dp = mfma32(QT::frag_rows(sdo, qt * 32, ks, lane), vf[ks], dp);
+        }
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int ql = qt * 32 + g * 8 + 4 * (lane >> 5);  // block-local first query of the group
+          const f32x4 l4 = *reinterpret_cast<const f32x4*>(sstat + ql);
+          const f32x4 d4 = *reinterpret_cast<const f32x4*>(sstat + 64 + ql);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int qi = qb + ql + e;
+            float x = s[g * 4 + e] * p.scale_log2;
+            if (HAS_BIAS)
+              x += (float)((const T*)p.bias)[(int64_t)h * p.bias_sh + (int64_t)qi * p.bias_sr + mykey] * kLog2e;
+            float pr = fast_exp2(x - l4[e]);
+            if (diag && mykey > qi) pr = 0.f;
+            s[g * 4 + e] = pr;
+            dp[g * 4 + e] = pr * (dp[g * 4 + e] - d4[e]);
+          }
+        }
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          const v8 pa = round8<T>(s, t);
+          const v8 dsa = round8<T>(dp, t);
+#pragma unroll
+          for (int d = 0; d < DT; ++d) {
+            dv[d] = mfma32(QT::frag_hd(sdo, qt * 32 + t * 16, d, lane), pa, dv[d]);
+            dk[d] = mfma32(QT::frag_hd(sq, qt * 32 + t * 16, d, lane), dsa, dk[d]);
+          }
+        }
+      }
+    }
+    if (more) commit(smem + ((it + 1) & 1) * STAGE);
+    __syncthreads();
+  }
+
+  if (active) {
+    T* dK = (T*)p.dk + base;
+    T* dV = (T*)p.dv + base;
+#pragma unroll
+    for (int d = 0; d < DT; ++d)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        v4 a, c;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          a[e] = (T)(dk[d][g * 4 + e] * p.scale);
+          c[e] = (T)dv[d][g * 4 + e];
+        }
+        const int64_t off = (int64_t)mykey * p.ss + d * 32 + g * 8 + 4 * (lane >> 5);
+        *reinterpret_cast<v4*>(dK + off) = a;
+        *reinterpret_cast<v4*>(dV + off) = c;
+      }
+  }
+}
+
+// ===========================================================================
+// dQ pass.  Workgroup: 4 waves x 32 queries; key/value blocks of 64 up to the
+// diagonal, K and V tiles through LDS.
+// ===========================================================================
+template <typename T, int HD, bool HAS_BIAS>
+__global__ __launch_bounds__(256) void attn_dq_kernel(AttnParams p) {
+  typedef SeqTile<T, 64, HD> KT;
+  typedef typename Vec<T>::v8 v8;
+  typedef typename Vec<T>::v4 v4;
+  constexpr int KS = HD / 16, DT = HD / 32;
+  constexpr int STAGE = 2 * KT::BYTES;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nbh = p.B * p.nh;
+  const int nqb = (p.S + 127) / 128;
+  const int qblk = nqb - 1 - (int)(blockIdx.x / nbh);
+  const int bh = blockIdx.x % nbh;
+  const int b = bh / p.nh, h = bh % p.nh;
+  const int64_t base = (int64_t)b * p.sb + (int64_t)h * p.sh;
+  const T* Q = (const T*)p.q + base;
+  const T* K = (const T*)p.k + base;
+  const T* V = (const T*)p.v + base;
+  const T* dO = (const T*)p.d_o + base;
+
+  const int q0 = qblk * 128;
+  const int q0w = q0 + wave * 32;
+  const bool active = q0w < p.S;
+  const int myq = q0w + (lane & 31);
+  const int kv_end = min(p.S, q0 + 128);
+  const int nkv = kv_end / 64;
+
+  v8 qf[KS], dof[KS];
+  float my_lse = 0.f, my_delta = 0.f;
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    u32x4 a = {0u, 0u, 0u, 0u}, c = {0u, 0u, 0u, 0u};
+    if (active) {
+      a = ld16(Q + (int64_t)myq * p.ss + ks * 16 + (lane >> 5) * 8);
+      c = ld16(dO + (int64_t)myq * p.ss + ks * 16 + (lane >> 5) * 8);
+    }
+    qf[ks] = __builtin_bit_cast(v8, a);
+    dof[ks] = __builtin_bit_cast(v8, c);
+  }
+  if (active) {
+    my_lse = p.lse[(int64_t)bh * p.S + myq];
+    my_delta = p.delta[(int64_t)bh * p.S + myq];
+  }
+  f32x16 dq[DT];
+#pragma unroll
+  for (int d = 0; d < DT; ++d)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dq[d][r] = 0.f;
+
+  u32x4 rk[KT::PER_THREAD], rv[KT::PER_THREAD];
+  KT::fetch(rk, K, p.ss, 0);
+  KT::fetch(rv, V, p.ss, 0);
+  KT::commit(smem, rk);
+  KT::commit(smem + KT::BYTES, rv);
+  __syncthreads();
+
+  for (int j = 0; j < nkv; ++j) {
+    const char* sk = smem + (j & 1) * STAGE;
+    const char* sv = sk + KT::BYTES;
+    const bool more = j + 1 < nkv;
+    if (more) {
+      KT::fetch(rk, K, p.ss, (j + 1) * 64);
+      KT::fetch(rv, V, p.ss, (j + 1) * 64);
+    }
+    const int kb = j * 64;
+    if (active) {
+#pragma unroll
+      for (int jt = 0; jt < 2; ++jt) {
+        const int ks0 = kb + jt * 32;  // first key of this 32-key sub-tile
+        if (ks0 > q0w + 31) continue;
+        const bool diag = ks0 + 31 > q0w;
+        f32x16 s, dp;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          s = mfma32(KT::frag_rows(sk, jt * 32, ks, lane), qf[ks], s);
+          dp = mfma32(KT::frag_rows(sv, jt * 32, ks, lane), dof[ks], dp);
+        }
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int key0 = ks0 + g * 8 + 4 * (lane >> 5);
+          float bv[4] = {0.f, 0.f, 0.f, 0.f};
+          if (HAS_BIAS) {
+            const v4 raw = *reinterpret_cast<const v4*>((const T*)p.bias + (int64_t)h * p.bias_sh +
+                                                        (int64_t)myq * p.bias_sr + key0);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) bv[e] = (float)raw[e] * kLog2e;
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            float pr = fast_exp2(s[g * 4 + e] * p.scale_log2 + bv[e] - my_lse);
+            if (diag && key0 + e > myq) pr = 0.f;
+            dp[g * 4 + e] = pr * (dp[g * 4 + e] - my_delta);
+          }
+        }
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          const v8 dsb = round8<T>(dp, t);
+#pragma unroll
+          for (int d = 0; d < DT; ++d) dq[d] = mfma32(KT::frag_hd(sk, jt * 32 + t * 16, d, lane), dsb, dq[d]);
+        }
+      }
+    }
+    if (more) {
+      char* dst = smem + ((j + 1) & 1) * STAGE;
+      KT::commit(dst, rk);
+      KT::commit(dst + KT::BYTES, rv);
+    }
+    __syncthreads();
+  }
+
+  if (active) {
+    T* dQ = (T*)p.dq + base;
+#pragma unroll
+    for (int d = 0; d < DT; ++d)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        v4 a;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) a[e] = (T)(dq[d][g * 4 + e] * p.scale);
+        *reinterpret_cast<v4*>(dQ + (int64_t)myq * p.ss + d * 32 + g * 8 + 4 * (lane >> 5)) = a;
+      }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// host dispatch
+// ---------------------------------------------------------------------------
+template <typename K>
+static void allow_lds(K kernel, int bytes) {
+  if (bytes > 64 * 1024)
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+}
+
+template <typename T, int HD, bool HB>
+static int fwd_launch(hipStream_t st, const AttnParams& p) {
+  constexpr int lds = 4 * SeqTile<T, 64, HD>::BYTES;
+  auto kernel = attn_fwd_kernel<T, HD, HB>;
+  static bool once = (allow_lds(kernel, lds), true);
+  (void)once;
+  const unsigned grid = (unsigned)(((p.S + 127) / 128) * p.B * p.nh);
+  kernel<<<dim3(grid), dim3(256), lds, st>>>(p);
+  TF_CHECK_LAUNCH();
+  return TF_OK;
+}
+
+template <typename T, int HD, bool HB>
+static int bwd_launch(hipStream_t st, const AttnParams& p) {
+  const int64_t rows = (int64_t)p.B * p.nh * p.S;
+  constexpr int rpb = 256 / (HD / 8);
+  attn_delta_kernel<T, HD><<<dim3((unsigned)((rows + rpb - 1) / rpb)), dim3(256), 0, st>>>(p);
+  TF_CHECK_LAUNCH();
+  const unsigned grid = (unsigned)(((p.S + 127) / 128) * p.B * p.nh);
+  {
+    constexpr int lds = 2 * (2 * SeqTile<T, 64, HD>::BYTES + 2 * 64 * 4);
+    auto kernel = attn_dkdv_kernel<T, HD, HB>;
+    static bool once = (allow_lds(kernel, lds), true);
+    (void)once;
+    kernel<<<dim3(grid), dim3(256), lds, st>>>(p);
+    TF_CHECK_LAUNCH();
+  }
+  {
+    constexpr int lds = 4 * SeqTile<T, 64, HD>::BYTES;
+    auto kernel = attn_dq_kernel<T, HD, HB>;
+    static bool once = (allow_lds(kernel, lds), true);
+    (void)once;
+    kernel<<<dim3(grid), dim3(256), lds, st>>>(p);
+    TF_CHECK_LAUNCH();
+  }
+  return TF_OK;
+}
+
+template <typename T, bool FWD>
+static int attn_dispatch(hipStream_t st, int hd, bool has_bias, const AttnParams& p) {
+#define GO(HD)                                                                          \
+  return FWD ? (has_bias ? fwd_launch<T, HD, true>(st, p) : fwd_launch<T, HD, false>(st, p)) \
+             : (has_bias ? bwd_launch<T, HD, true>(st, p) : bwd_launch<T, HD, false>(st, p))
+  switch (hd) {
+    case 32: GO(32);
+    case 64: GO(64);
+    case 128: GO(128);
+  }
+#undef GO
+  return TF_ESHAPE;
+}
+
+static int attn_check(int dtype, int64_t B, int64_t nh, int64_t S, int64_t hd, int64_t sb, int64_t sh, int64_t ss,
+                      const void* bias, int64_t bias_sh, int64_t bias_sr) {
+  if (dtype != TF_F16 && dtype != TF_BF16) return TF_EDTYPE;
+  if (B <= 0 || nh <= 0 || S <= 0) return TF_EINVAL;
+  if (hd != 32 && hd != 64 && hd != 128) return TF_ESHAPE;  // as kernels/attention.py:567
+  if (S % 64 != 0) return TF_ESHAPE;                        // as kernels/attention.py:181-183
+  if (B * nh * ((S + 127) / 128) > 0x7fffffff || S > (1 << 24)) return TF_EINVAL;
+  if (sb % 8 || sh % 8 || ss % 8 || ss < hd) return TF_EALIGN;
+  if (bias && (bias_sh % 4 || bias_sr % 4 || bias_sr < S)) return TF_EALIGN;
+  return TF_OK;
+}
+
+}  // namespace tfa
+
+using namespace tfa;
+
+extern "C" int tf_attn_fwd(void* stream, int dtype, int64_t B, int64_t nh, int64_t S, int64_t hd, const void* q,
+                           const void* k, const void* v, void* o, int64_t sb, int64_t sh, int64_t ss, float* lse,
+                           const void* bias, int64_t bias_sh, int64_t bias_sr, float scale) {
+  if (!q || !k || !v || !o || !lse) return TF_EINVAL;
+  const int rc = attn_check(dtype, B, nh, S, hd, sb, sh, ss, bias, bias_sh, bias_sr);
+  if (rc != TF_OK) return rc;
+  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o)) return TF_EALIGN;
+  if (bias && (reinterpret_cast<uintptr_t>(bias) & 7)) return TF_EALIGN;
+  AttnParams p = {};
+  p.q = q; p.k = k; p.v = v; p.out = o; p.lse = lse; p.bias = bias;
+  p.sb = sb; p.sh = sh; p.ss = ss; p.bias_sh = bias_sh; p.bias_sr = bias_sr;
+  p.B = (int)B; p.nh = (int)nh; p.S = (int)S;
+  p.scale = scale; p.scale_log2 = scale * kLog2e;
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == TF_F16) return attn_dispatch<f16, true>(st, (int)hd, bias != nullptr, p);
+  return attn_dispatch<bf16, true>(st, (int)hd, bias != nullptr, p);
+}
+
+extern "C" int tf_attn_bwd(void* stream, int dtype, int64_t B, int64_t nh, int64_t S, int64_t hd, const void* q,
+                           const void* k, const void* v, const void* o, const void* d_o, void* dq, void* dk, void* dv,
+                           int64_t sb, int64_t sh, int64_t ss, const float* lse, float* delta, const void* bias,
+                           int64_t bias_sh, int64_t bias_sr, float scale) {
+  if (!q || !k || !v || !o || !d_o || !dq || !dk || !dv || !lse || !delta) return TF_EINVAL;
+  const int rc = attn_check(dtype, B, nh, S, hd, sb, sh, ss, bias, bias_sh, bias_sr);
+  if (rc != TF_OK) return rc;
+  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o) || !aligned16(d_o) || !aligned16(dq) ||
+      !aligned16(dk) || !aligned16(dv))
+    return TF_EALIGN;
+  if (bias && (reinterpret_cast<uintptr_t>(bias) & 7)) return TF_EALIGN;
+  AttnParams p = {};
+  p.q = q; p.k = k; p.v = v; p.o = o; p.d_o = d_o; p.dq = dq; p.dk = dk; p.dv = dv;
+  p.lse = const_cast<float*>(lse); p.delta = delta; p.bias = bias;
+  p.sb = sb; p.sh = sh; p.ss = ss; p.bias_sh = bias_sh; p.bias_sr = bias_sr;
+  p.B = (int)B; p.nh = (int)nh; p.S = (int)S;
+  p.scale = scale; p.scale_log2 = scale * kLog2e;
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == TF_F16) return attn_dispatch<f16, false>(st, (int)hd, bias != nullptr, p);
+  return attn_dispatch<bf16, false>(st, (int)hd, bias != nullptr, p);
+}

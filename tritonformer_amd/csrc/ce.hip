@@ -1,0 +1,171 @@
+// Cross-entropy forward/backward for gfx950.  HBM-bound: the forward streams
+// each logits row once (online max / sum-of-exp in the log2 domain), the
+// backward streams it once more and writes the gradient, already multiplied by
+// the upstream per-row gradient.
+#include "rowops.h"
+
+namespace tfa {
+
+constexpr int kCeThreads = 256;
+
+struct MaxSum {
+  float m;  // running max of x*log2e
+  float s;  // running sum of exp2(x*log2e - m)
+};
+__device__ __forceinline__ MaxSum combine(MaxSum a, MaxSum b) {
+  const float m = fmaxf(a.m, b.m);
+  MaxSum r;
+  r.m = m;
+  // exp2f(-inf - finite) = 0; both -inf only when both are empty (s = 0).
+  r.s = (m == -INFINITY) ? 0.f : a.s * exp2f(a.m - m) + b.s * exp2f(b.m - m);
+  return r;
+}
+
+__device__ __forceinline__ MaxSum block_combine(MaxSum v, MaxSum* smem) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    MaxSum other;
+    other.m = __shfl_xor(v.m, o, 64);
+    other.s = __shfl_xor(v.s, o, 64);
+    v = combine(v, other);
+  }
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) smem[wave] = v;
+  __syncthreads();
+  MaxSum r = smem[0];
+#pragma unroll
+  for (int w = 1; w < kCeThreads / 64; ++w) r = combine(r, smem[w]);
+  return r;
+}
+
+template <typename T, bool VEC>
+__global__ __launch_bounds__(kCeThreads) void ce_fwd(int V, const T* __restrict__ logits, int64_t ld,
+                                                      const int64_t* __restrict__ labels, T* __restrict__ loss,
+                                                      float* __restrict__ lse) {
+  __shared__ MaxSum smem[kCeThreads / 64];
+  const int64_t row = blockIdx.x;
+  const T* xr = logits + row * ld;
+  MaxSum acc = {-INFINITY, 0.f};
+  if (VEC) {
+    const int nchunk = V >> 3;
+    for (int c = threadIdx.x; c < nchunk; c += kCeThreads) {
+      float v[8];
+      Chunk<T>::load(xr + c * 8, v);
+      float cm = v[0];
+#pragma unroll
+      for (int e = 1; e < 8; ++e) cm = fmaxf(cm, v[e]);
+      cm *= kLog2e;
+      if (cm > acc.m) { acc.s *= exp2f(acc.m - cm); acc.m = cm; }
+      float part = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) part += exp2f(v[e] * kLog2e - acc.m);
+      acc.s += part;
+    }
+  } else {
+    for (int c = threadIdx.x; c < V; c += kCeThreads) {
+      const float t = (float)xr[c] * kLog2e;
+      if (t > acc.m) { acc.s *= exp2f(acc.m - t); acc.m = t; }
+      acc.s += exp2f(t - acc.m);
+    }
+  }
+  const MaxSum tot = block_combine(acc, smem);
+  if (threadIdx.x == 0) {
+    const float l = (tot.m + log2f(tot.s)) * kLn2;  // natural-log logsumexp
+    lse[row] = l;
+    const int64_t lab = labels[row];
+    const float xl = (lab >= 0 && lab < V) ? (float)xr[lab] : 0.f;
+    loss[row] = (T)(l - xl);
+  }
+}
+
+template <typename T, bool VEC>
+__global__ __launch_bounds__(kCeThreads) void ce_bwd(int V, const T* __restrict__ logits, int64_t ld,
+                                                      const int64_t* __restrict__ labels,
+                                                      const float* __restrict__ lse, const T* __restrict__ gout,
+                                                      int64_t gstride, T* __restrict__ dlogits, int64_t ldd) {
+  const int64_t row = blockIdx.x;
+  const T* xr = logits + row * ld;
+  T* dr = dlogits + row * ldd;
+  const float l2 = lse[row] * kLog2e;
+  const float g = (float)gout[row * gstride];
+  const int lab = (int)labels[row];
+  if (VEC) {
+    const int nchunk = V >> 3;
+    for (int c = threadIdx.x; c < nchunk; c += kCeThreads) {
+      float v[8];
+      Chunk<T>::load(xr + c * 8, v);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = exp2f(v[e] * kLog2e - l2);
+      if ((lab >> 3) == c) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] -= (e == (lab & 7)) ? 1.0f : 0.0f;
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] *= g;
+      Chunk<T>::store(dr + c * 8, v);
+    }
+  } else {
+    for (int c = threadIdx.x; c < V; c += kCeThreads) {
+      float p = exp2f((float)xr[c] * kLog2e - l2);
+      if (c == lab) p -= 1.0f;
+      dr[c] = (T)(p * g);
+    }
+  }
+}
+
+template <typename T>
+static int ce_fwd_launch(hipStream_t st, int64_t rows, int64_t V, const void* logits, int64_t ld,
+                         const int64_t* labels, void* loss, float* lse) {
+  const dim3 grid((unsigned)rows), block(kCeThreads);
+  if (row_vectorizable<T>(logits, V, ld))
+    ce_fwd<T, true><<<grid, block, 0, st>>>((int)V, (const T*)logits, ld, labels, (T*)loss, lse);
+  else
+    ce_fwd<T, false><<<grid, block, 0, st>>>((int)V, (const T*)logits, ld, labels, (T*)loss, lse);
+  TF_CHECK_LAUNCH();
+  return TF_OK;
+}
+
+template <typename T>
+static int ce_bwd_launch(hipStream_t st, int64_t rows, int64_t V, const void* logits, int64_t ld,
+                         const int64_t* labels, const float* lse, const void* gout, int64_t gstride,
+                         void* dlogits, int64_t ldd) {
+  const dim3 grid((unsigned)rows), block(kCeThreads);
+  if (row_vectorizable<T>(logits, V, ld) && row_vectorizable<T>(dlogits, V, ldd))
+    ce_bwd<T, true><<<grid, block, 0, st>>>((int)V, (const T*)logits, ld, labels, lse, (const T*)gout, gstride,
+                                            (T*)dlogits, ldd);
+  else
+    ce_bwd<T, false><<<grid, block, 0, st>>>((int)V, (const T*)logits, ld, labels, lse, (const T*)gout, gstride,
+                                             (T*)dlogits, ldd);
+  TF_CHECK_LAUNCH();
+  return TF_OK;
+}
+
+}  // namespace tfa
+
+using namespace tfa;
+
+extern "C" int tf_cross_entropy_fwd(void* stream, int dtype, int64_t rows, int64_t V, const void* logits,
+                                    int64_t ld, const int64_t* labels, void* loss, float* lse) {
+  if (!logits || !labels || !loss || !lse) return TF_EINVAL;
+  if (rows < 0 || rows > 0x7fffffff || V <= 0 || V > (1 << 30) || ld < V) return TF_EINVAL;
+  if (rows == 0) return TF_OK;
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == TF_F16) return ce_fwd_launch<f16>(st, rows, V, logits, ld, labels, loss, lse);
+  if (dtype == TF_BF16) return ce_fwd_launch<bf16>(st, rows, V, logits, ld, labels, loss, lse);
+  return TF_EDTYPE;
+}
+
+extern "C" int tf_cross_entropy_bwd(void* stream, int dtype, int64_t rows, int64_t V, const void* logits,
+                                    int64_t ld, const int64_t* labels, const float* lse, const void* gout,
+                                    int64_t gout_stride, void* dlogits, int64_t ldd) {
+  if (!logits || !labels || !lse || !gout || !dlogits) return TF_EINVAL;
+  if (rows < 0 || rows > 0x7fffffff || V <= 0 || V > (1 << 30) || ld < V || ldd < V || gout_stride < 0)
+    return TF_EINVAL;
+  if (rows == 0) return TF_OK;
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == TF_F16)
+    return ce_bwd_launch<f16>(st, rows, V, logits, ld, labels, lse, gout, gout_stride, dlogits, ldd);
+  if (dtype == TF_BF16)
+    return ce_bwd_launch<bf16>(st, rows, V, logits, ld, labels, lse, gout, gout_stride, dlogits, ldd);
+  return TF_EDTYPE;
+}

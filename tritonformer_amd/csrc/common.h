@@ -1,0 +1,92 @@
+// Shared device helpers for the gfx950 kernels: 16-bit types, 16-byte vector
+// access, wave64 reductions and MFMA wrappers.  gfx950 only, wave size 64.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "../../include/tritonformer_amd.h"
+
+namespace tfa {
+
+typedef _Float16 f16;
+typedef __bf16 bf16;
+
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+template <typename T> struct Vec;
+template <> struct Vec<f16> { typedef f16x8 v8; typedef f16x4 v4; };
+template <> struct Vec<bf16> { typedef bf16x8 v8; typedef bf16x4 v4; };
+
+template <typename T> __device__ __forceinline__ float to_f32(T v) { return (float)v; }
+template <typename T> __device__ __forceinline__ T from_f32(float v) { return (T)v; }
+
+// ---- wave64 reductions (butterfly over cross-lane shuffles) ---------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+// ---- 16-byte global access -------------------------------------------------
+__device__ __forceinline__ u32x4 ld16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
+__device__ __forceinline__ void st16(void* p, u32x4 v) { *reinterpret_cast<u32x4*>(p) = v; }
+
+template <typename T> __device__ __forceinline__ void unpack8(u32x4 raw, float (&out)[8]) {
+  typename Vec<T>::v8 h = __builtin_bit_cast(typename Vec<T>::v8, raw);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) out[i] = (float)h[i];
+}
+template <typename T> __device__ __forceinline__ u32x4 pack8(const float (&in)[8]) {
+  typename Vec<T>::v8 h;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) h[i] = (T)in[i];
+  return __builtin_bit_cast(u32x4, h);
+}
+
+// ---- MFMA 32x32x16, D(32x32 fp32) += A(32x16) * B(16x32) ------------------
+// Lane l supplies A[l%32][(l/32)*8 .. +8] and B[(l/32)*8 .. +8][l%32];
+// result register r of lane l is D[(r/4)*8 + (l/32)*4 + r%4][l%32].
+__device__ __forceinline__ f32x16 mfma32(f16x8 a, f16x8 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+
+// ---- LDS access ------------------------------------------------------------
+typedef __attribute__((address_space(3))) void lds_void;
+
+__device__ __forceinline__ u32x4 lds_ld16(const char* base, int byte_off) {
+  return *reinterpret_cast<const u32x4*>(base + byte_off);
+}
+__device__ __forceinline__ void lds_st16(char* base, int byte_off, u32x4 v) {
+  *reinterpret_cast<u32x4*>(base + byte_off) = v;
+}
+// Transposing 8-byte LDS read: within each group of 16 lanes, lane i supplies
+// the address of 4 consecutive 16-bit elements; viewing the 16 loads as a
+// 4x16 matrix (row = i/4, 4 columns per lane), lane j receives column j.
+__device__ __forceinline__ u32x2 lds_ld8_tr(const char* base, int byte_off) {
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(base + byte_off));
+  return __builtin_bit_cast(u32x2, v);
+}
+
+inline int ceil_div(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
+
+}  // namespace tfa

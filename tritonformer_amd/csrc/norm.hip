@@ -1,0 +1,524 @@
+// LayerNorm forward/backward and row softmax forward/backward for gfx950.
+// All four are HBM-bound: one wave64 owns one row, holds it in registers as
+// 16-byte chunks (chunk c of the row belongs to lane c % 64), and reduces with
+// cross-lane shuffles, so every element is read from HBM exactly once.
+#include "rowops.h"
+
+namespace tfa {
+
+constexpr int kRowsPerBlock = 4;  // 4 waves per workgroup, one row each
+
+// ---------------------------------------------------------------------------
+// LayerNorm forward.  NV = 16-byte chunks per lane (row length <= NV*64*8).
+// ---------------------------------------------------------------------------
+template <typename T, int NV>
+__global__ __launch_bounds__(256) void ln_fwd_vec(int64_t rows, int d, const T* __restrict__ x, int64_t ldx,
+                                                   const T* __restrict__ gamma, const T* __restrict__ beta,
+                                                   float eps, T* __restrict__ y, int64_t ldy,
+                                                   float* __restrict__ mean_out, float* __restrict__ rstd_out) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int nchunk = d >> 3;
+  const T* xr = x + row * ldx;
+  float v[NV][8];
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = lane + i * 64;
+    if (c < nchunk) {
+      Chunk<T>::load(xr + c * 8, v[i]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) s += v[i][e];
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[i][e] = 0.f;
+    }
+  }
+  const float mean = wave_sum(s) / (float)d;
+  float q = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    if (lane + i * 64 < nchunk) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { const float t = v[i][e] - mean; q += t * t; }
+    }
+  }
+  const float var = wave_sum(q) / (float)d;
+  const float rstd = 1.0f / sqrtf(var + eps);
+  if (lane == 0) { mean_out[row] = mean; rstd_out[row] = rstd; }
+  T* yr = y + row * ldy;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = lane + i * 64;
+    if (c < nchunk) {
+      float g[8], b[8], o[8];
+      Chunk<T>::load(gamma + c * 8, g);
+      Chunk<T>::load(beta + c * 8, b);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[e] = (v[i][e] - mean) * rstd * g[e] + b[e];
+      Chunk<T>::store(yr + c * 8, o);
+    }
+  }
+}
+
+// Any row length / alignment: scalar loads, three passes over the row (the
+// second and third come from cache).
+template <typename T>
+__global__ __launch_bounds__(256) void ln_fwd_any(int64_t rows, int d, const T* __restrict__ x, int64_t ldx,
+                                                   const T* __restrict__ gamma, const T* __restrict__ beta,
+                                                   float eps, T* __restrict__ y, int64_t ldy,
+                                                   float* __restrict__ mean_out, float* __restrict__ rstd_out) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const T* xr = x + row * ldx;
+  float s = 0.f;
+  for (int c = lane; c < d; c += 64) s += (float)xr[c];
+  const float mean = wave_sum(s) / (float)d;
+  float q = 0.f;
+  for (int c = lane; c < d; c += 64) { const float t = (float)xr[c] - mean; q += t * t; }
+  const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)d + eps);
+  if (lane == 0) { mean_out[row] = mean; rstd_out[row] = rstd; }
+  T* yr = y + row * ldy;
+  for (int c = lane; c < d; c += 64)
+    yr[c] = (T)(((float)xr[c] - mean) * rstd * (float)gamma[c] + (float)beta[c]);
+}
+
+// ---------------------------------------------------------------------------
+// LayerNorm backward.  Wave w of workgroup b walks rows (b*4 + w) + k*4*grid.
+// dx is written per row; dgamma/dbeta partial sums stay in registers, are
+// summed over the 4 waves through LDS and land in partial[b][0|1][d].
+// ---------------------------------------------------------------------------
+template <typename T, int NV>
+__global__ __launch_bounds__(256) void ln_bwd_vec(int64_t rows, int d, const T* __restrict__ dy, int64_t lddy,
+                                                   const T* __restrict__ x, int64_t ldx,
+                                                   const T* __restrict__ gamma, const float* __restrict__ mean,
+                                                   const float* __restrict__ rstd, T* __restrict__ dx,
+                                                   int64_t lddx, float* __restrict__ partial) {
+  extern __shared__ float red[];  // [4][d]
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int nchunk = d >> 3;
+  float g[NV][8], dg[NV][8], db[NV][8];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = lane + i * 64;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { dg[i][e] = 0.f; db[i][e] = 0.f; g[i][e] = 0.f; }
+    if (c < nchunk) Chunk<T>::load(gamma + c * 8, g[i]);
+  }
+  const float inv_d = 1.0f / (float)d;
+  for (int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + wave; row < rows;
+       row += (int64_t)gridDim.x * kRowsPerBlock) {
+    const float mu = mean[row], rs = rstd[row];
+    const T* xr = x + row * ldx;
+    const T* dyr = dy + row * lddy;
+    float xh[NV][8], gd[NV][8];
+    float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int c = lane + i * 64;
+      if (c < nchunk) {
+        float xv[8], dv[8];
+        Chunk<T>::load(xr + c * 8, xv);
+        Chunk<T>::load(dyr + c * 8, dv);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          xh[i][e] = (xv[e] - mu) * rs;
+          gd[i][e] = dv[e] * g[i][e];
+          s1 += gd[i][e] * xh[i][e];
+          s2 += gd[i][e];
+          dg[i][e] += dv[e] * xh[i][e];
+          db[i][e] += dv[e];
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { xh[i][e] = 0.f; gd[i][e] = 0.f; }
+      }
+    }
+    const float c1 = wave_sum(s1) * inv_d;
+    const float c2 = wave_sum(s2) * inv_d;
+    T* dxr = dx + row * lddx;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int c = lane + i * 64;
+      if (c < nchunk) {
+        float o[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = (gd[i][e] - xh[i][e] * c1 - c2) * rs;
+        Chunk<T>::store(dxr + c * 8, o);
+      }
+    }
+  }
+  // cross-wave reduction, dgamma then dbeta, through one [4][d] LDS buffer
+  float* pout = partial + (int64_t)blockIdx.x * 2 * d;
+#pragma unroll
+  for (int which = 0; which < 2; ++which) {
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int c = lane + i * 64;
+      if (c < nchunk) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) red[wave * d + c * 8 + e] = which ? db[i][e] : dg[i][e];
+      }
+    }
+    __syncthreads();
+    for (int c = threadIdx.x; c < d; c += 256)
+      pout[which * d + c] = red[c] + red[d + c] + red[2 * d + c] + red[3 * d + c];
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void ln_bwd_any(int64_t rows, int d, const T* __restrict__ dy, int64_t lddy,
+                                                   const T* __restrict__ x, int64_t ldx,
+                                                   const T* __restrict__ gamma, const float* __restrict__ mean,
+                                                   const float* __restrict__ rstd, T* __restrict__ dx,
+                                                   int64_t lddx, float* __restrict__ partial) {
+  // One workgroup per slice of rows; every thread owns columns tid, tid+256, ...
+  // so the dgamma/dbeta partials need no cross-thread reduction; the per-row
+  // sums are reduced per wave, with all 4 waves walking the same row.
+  __shared__ float sred[2][4];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const float inv_d = 1.0f / (float)d;
+  float* pout = partial + (int64_t)blockIdx.x * 2 * d;
+  for (int c = threadIdx.x; c < d; c += 256) { pout[c] = 0.f; pout[d + c] = 0.f; }
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    const float mu = mean[row], rs = rstd[row];
+    const T* xr = x + row * ldx;
+    const T* dyr = dy + row * lddy;
+    float s1 = 0.f, s2 = 0.f;
+    for (int c = threadIdx.x; c < d; c += 256) {
+      const float xh = ((float)xr[c] - mu) * rs, dv = (float)dyr[c], gd = dv * (float)gamma[c];
+      s1 += gd * xh;
+      s2 += gd;
+      pout[c] += dv * xh;
+      pout[d + c] += dv;
+    }
+    s1 = wave_sum(s1);
+    s2 = wave_sum(s2);
+    __syncthreads();
+    if (lane == 0) { sred[0][wave] = s1; sred[1][wave] = s2; }
+    __syncthreads();
+    const float c1 = (sred[0][0] + sred[0][1] + sred[0][2] + sred[0][3]) * inv_d;
+    const float c2 = (sred[1][0] + sred[1][1] + sred[1][2] + sred[1][3]) * inv_d;
+    T* dxr = dx + row * lddx;
+    for (int c = threadIdx.x; c < d; c += 256) {
+      const float xh = ((float)xr[c] - mu) * rs, gd = (float)dyr[c] * (float)gamma[c];
+      dxr[c] = (T)((gd - xh * c1 - c2) * rs);
+    }
+  }
+}
+
+// Second stage: dgamma[c] = sum_b partial[b][0][c], dbeta[c] = sum_b partial[b][1][c].
+// Workgroup = 64 columns x 4 slices of the partial rows.
+template <typename T>
+__global__ __launch_bounds__(256) void ln_bwd_reduce(int nparts, int d, const float* __restrict__ partial,
+                                                      T* __restrict__ dgamma, T* __restrict__ dbeta) {
+  __shared__ float red[2][4][64];
+  const int col = blockIdx.x * 64 + (threadIdx.x & 63);
+  const int slice = threadIdx.x >> 6;
+  float a = 0.f, b = 0.f;
+  if (col < d) {
+    for (int p = slice; p < nparts; p += 4) {
+      a += partial[(int64_t)p * 2 * d + col];
+      b += partial[(int64_t)p * 2 * d + d + col];
+    }
+  }
+  red[0][slice][threadIdx.x & 63] = a;
+  red[1][slice][threadIdx.x & 63] = b;
+  __syncthreads();
+  if (slice == 0 && col < d) {
+    const int l = threadIdx.x;
+    dgamma[col] = (T)(red[0][0][l] + red[0][1][l] + red[0][2][l] + red[0][3][l]);
+    dbeta[col] = (T)(red[1][0][l] + red[1][1][l] + red[1][2][l] + red[1][3][l]);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Softmax (T = f16 / bf16 / float).  NV chunks of Chunk<T>::N elements per lane.
+// ---------------------------------------------------------------------------
+template <typename T, int NV>
+__global__ __launch_bounds__(256) void softmax_fwd_vec(int64_t rows, int cols, const T* __restrict__ x,
+                                                        int64_t ldx, T* __restrict__ y, int64_t ldy) {
+  constexpr int N = Chunk<T>::N;
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int nchunk = cols / N;
+  const T* xr = x + row * ldx;
+  float v[NV][N];
+  float m = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = lane + i * 64;
+    if (c < nchunk) {
+      Chunk<T>::load(xr + c * N, v[i]);
+#pragma unroll
+      for (int e = 0; e < N; ++e) m = fmaxf(m, v[i][e]);
+    }
+  }
+  m = wave_max(m);
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    if (lane + i * 64 < nchunk) {
+#pragma unroll
+      for (int e = 0; e < N; ++e) { v[i][e] = exp2f((v[i][e] - m) * kLog2e); s += v[i][e]; }
+    }
+  }
+  const float inv = 1.0f / wave_sum(s);
+  T* yr = y + row * ldy;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = lane + i * 64;
+    if (c < nchunk) {
+#pragma unroll
+      for (int e = 0; e < N; ++e) v[i][e] *= inv;
+      Chunk<T>::store(yr + c * N, v[i]);
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void softmax_fwd_any(int64_t rows, int cols, const T* __restrict__ x,
+                                                        int64_t ldx, T* __restrict__ y, int64_t ldy) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const T* xr = x + row * ldx;
+  float m = -INFINITY;
+  for (int c = lane; c < cols; c += 64) m = fmaxf(m, (float)xr[c]);
+  m = wave_max(m);
+  float s = 0.f;
+  for (int c = lane; c < cols; c += 64) s += exp2f(((float)xr[c] - m) * kLog2e);
+  const float inv = 1.0f / wave_sum(s);
+  T* yr = y + row * ldy;
+  for (int c = lane; c < cols; c += 64) yr[c] = (T)(exp2f(((float)xr[c] - m) * kLog2e) * inv);
+}
+
+template <typename T, int NV>
+__global__ __launch_bounds__(256) void softmax_bwd_vec(int64_t rows, int cols, const T* __restrict__ dy,
+                                                        int64_t lddy, const T* __restrict__ y, int64_t ldy,
+                                                        T* __restrict__ dx, int64_t lddx) {
+  constexpr int N = Chunk<T>::N;
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int nchunk = cols / N;
+  float yv[NV][N], gv[NV][N];
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = lane + i * 64;
+    if (c < nchunk) {
+      Chunk<T>::load(y + row * ldy + c * N, yv[i]);
+      Chunk<T>::load(dy + row * lddy + c * N, gv[i]);
+#pragma unroll
+      for (int e = 0; e < N; ++e) s += yv[i][e] * gv[i][e];
+    }
+  }
+  s = wave_sum(s);
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = lane + i * 64;
+    if (c < nchunk) {
+      float o[N];
+#pragma unroll
+      for (int e = 0; e < N; ++e) o[e] = yv[i][e] * (gv[i][e] - s);
+      Chunk<T>::store(dx + row * lddx + c * N, o);
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void softmax_bwd_any(int64_t rows, int cols, const T* __restrict__ dy,
+                                                        int64_t lddy, const T* __restrict__ y, int64_t ldy,
+                                                        T* __restrict__ dx, int64_t lddx) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  float s = 0.f;
+  for (int c = lane; c < cols; c += 64) s += (float)y[row * ldy + c] * (float)dy[row * lddy + c];
+  s = wave_sum(s);
+  for (int c = lane; c < cols; c += 64)
+    dx[row * lddx + c] = (T)((float)y[row * ldy + c] * ((float)dy[row * lddy + c] - s));
+}
+
+// ---------------------------------------------------------------------------
+// host dispatch
+// ---------------------------------------------------------------------------
+static int pick_nv(int64_t nchunk) {
+  if (nchunk <= 64) return 1;
+  if (nchunk <= 128) return 2;
+  if (nchunk <= 256) return 4;
+  if (nchunk <= 512) return 8;
+  return 0;
+}
+
+template <typename T>
+static int ln_fwd_launch(hipStream_t st, int64_t rows, int64_t d, const void* x, int64_t ldx, const void* gamma,
+                         const void* beta, float eps, void* y, int64_t ldy, float* mean, float* rstd) {
+  const dim3 grid((unsigned)ceil_div(rows, kRowsPerBlock)), block(256);
+  const bool vec = row_vectorizable<T>(x, d, ldx) && row_vectorizable<T>(y, d, ldy) && aligned16(gamma) &&
+                   aligned16(beta);
+  const int nv = vec ? pick_nv(d / 8) : 0;
+#define LN_FWD(NV)                                                                                           \
+  ln_fwd_vec<T, NV><<<grid, block, 0, st>>>(rows, (int)d, (const T*)x, ldx, (const T*)gamma, (const T*)beta, \
+                                            eps, (T*)y, ldy, mean, rstd)
+  switch (nv) {
+    case 1: LN_FWD(1); break;
+    case 2: LN_FWD(2); break;
+    case 4: LN_FWD(4); break;
+    case 8: LN_FWD(8); break;
+    default:
+      ln_fwd_any<T><<<grid, block, 0, st>>>(rows, (int)d, (const T*)x, ldx, (const T*)gamma, (const T*)beta, eps,
+                                            (T*)y, ldy, mean, rstd);
+  }
+#undef LN_FWD
+  TF_CHECK_LAUNCH();
+  return TF_OK;
+}
+
+static int ln_bwd_parts(int64_t rows) {
+  int64_t g = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
+  return (int)(g < 512 ? g : 512);
+}
+
+template <typename T>
+static int ln_bwd_launch(hipStream_t st, int64_t rows, int64_t d, const void* dy, int64_t lddy, const void* x,
+                         int64_t ldx, const void* gamma, const float* mean, const float* rstd, void* dx,
+                         int64_t lddx, void* dgamma, void* dbeta, float* partial) {
+  const int parts = ln_bwd_parts(rows);
+  const bool vec = row_vectorizable<T>(x, d, ldx) && row_vectorizable<T>(dy, d, lddy) &&
+                   row_vectorizable<T>(dx, d, lddx) && aligned16(gamma);
+  const int nv = vec ? pick_nv(d / 8) : 0;
+  const size_t lds = (size_t)4 * d * sizeof(float);
+#define LN_BWD(NV)                                                                                          \
+  ln_bwd_vec<T, NV><<<dim3(parts), dim3(256), lds, st>>>(rows, (int)d, (const T*)dy, lddy, (const T*)x, ldx, \
+                                                         (const T*)gamma, mean, rstd, (T*)dx, lddx, partial)
+  switch (nv) {
+    case 1: LN_BWD(1); break;
+    case 2: LN_BWD(2); break;
+    case 4: LN_BWD(4); break;
+    case 8: LN_BWD(8); break;
+    default:
+      ln_bwd_any<T><<<dim3(parts), dim3(256), 0, st>>>(rows, (int)d, (const T*)dy, lddy, (const T*)x, ldx,
+                                                       (const T*)gamma, mean, rstd, (T*)dx, lddx, partial);
+  }
+#undef LN_BWD
+  TF_CHECK_LAUNCH();
+  ln_bwd_reduce<T><<<dim3(ceil_div(d, 64)), dim3(256), 0, st>>>(parts, (int)d, partial, (T*)dgamma, (T*)dbeta);
+  TF_CHECK_LAUNCH();
+  return TF_OK;
+}
+
+template <typename T>
+static int softmax_fwd_launch(hipStream_t st, int64_t rows, int64_t cols, const void* x, int64_t ldx, void* y,
+                              int64_t ldy) {
+  const dim3 grid((unsigned)ceil_div(rows, kRowsPerBlock)), block(256);
+  const bool vec = row_vectorizable<T>(x, cols, ldx) && row_vectorizable<T>(y, cols, ldy);
+  const int nv = vec ? pick_nv(cols / Chunk<T>::N) : 0;
+#define SM_FWD(NV) softmax_fwd_vec<T, NV><<<grid, block, 0, st>>>(rows, (int)cols, (const T*)x, ldx, (T*)y, ldy)
+  switch (nv) {
+    case 1: SM_FWD(1); break;
+    case 2: SM_FWD(2); break;
+    case 4: SM_FWD(4); break;
+    case 8: SM_FWD(8); break;
+    default: softmax_fwd_any<T><<<grid, block, 0, st>>>(rows, (int)cols, (const T*)x, ldx, (T*)y, ldy);
+  }
+#undef SM_FWD
+  TF_CHECK_LAUNCH();
+  return TF_OK;
+}
+
+template <typename T>
+static int softmax_bwd_launch(hipStream_t st, int64_t rows, int64_t cols, const void* dy, int64_t lddy,
+                              const void* y, int64_t ldy, void* dx, int64_t lddx) {
+  const dim3 grid((unsigned)ceil_div(rows, kRowsPerBlock)), block(256);
+  const bool vec =
+      row_vectorizable<T>(dy, cols, lddy) && row_vectorizable<T>(y, cols, ldy) && row_vectorizable<T>(dx, cols, lddx);
+  const int nv = vec ? pick_nv(cols / Chunk<T>::N) : 0;
+#define SM_BWD(NV) \
+  softmax_bwd_vec<T, NV><<<grid, block, 0, st>>>(rows, (int)cols, (const T*)dy, lddy, (const T*)y, ldy, (T*)dx, lddx)
+  switch (nv) {
+    case 1: SM_BWD(1); break;
+    case 2: SM_BWD(2); break;
+    case 4: SM_BWD(4); break;
+    case 8: SM_BWD(8); break;
+    default:
+      softmax_bwd_any<T><<<grid, block, 0, st>>>(rows, (int)cols, (const T*)dy, lddy, (const T*)y, ldy, (T*)dx, lddx);
+  }
+#undef SM_BWD
+  TF_CHECK_LAUNCH();
+  return TF_OK;
+}
+
+static bool bad_rows(int64_t rows, int64_t n, int64_t ld) {
+  return rows < 0 || n <= 0 || n > (1 << 30) || ld < n || rows > (int64_t)kRowsPerBlock * 0x7fffffff;
+}
+
+}  // namespace tfa
+
+using namespace tfa;
+
+extern "C" int tf_layernorm_fwd(void* stream, int dtype, int64_t rows, int64_t d, const void* x, int64_t ldx,
+                                const void* gamma, const void* beta, float eps, void* y, int64_t ldy,
+                                float* mean, float* rstd) {
+  if (!x || !gamma || !beta || !y || !mean || !rstd) return TF_EINVAL;
+  if (bad_rows(rows, d, ldx) || ldy < d) return TF_EINVAL;
+  if (rows == 0) return TF_OK;
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == TF_F16) return ln_fwd_launch<f16>(st, rows, d, x, ldx, gamma, beta, eps, y, ldy, mean, rstd);
+  if (dtype == TF_BF16) return ln_fwd_launch<bf16>(st, rows, d, x, ldx, gamma, beta, eps, y, ldy, mean, rstd);
+  return TF_EDTYPE;
+}
+
+extern "C" int64_t tf_layernorm_bwd_partial_bytes(int64_t rows, int64_t d) {
+  if (rows <= 0 || d <= 0) return 0;
+  return (int64_t)ln_bwd_parts(rows) * 2 * d * (int64_t)sizeof(float);
+}
+
+extern "C" int tf_layernorm_bwd(void* stream, int dtype, int64_t rows, int64_t d, const void* dy, int64_t lddy,
+                                const void* x, int64_t ldx, const void* gamma, const float* mean,
+                                const float* rstd, void* dx, int64_t lddx, void* dgamma, void* dbeta,
+                                float* partial, int64_t partial_bytes) {
+  if (!dy || !x || !gamma || !mean || !rstd || !dx || !dgamma || !dbeta) return TF_EINVAL;
+  if (bad_rows(rows, d, ldx) || lddy < d || lddx < d || rows == 0) return TF_EINVAL;
+  if (!partial || partial_bytes < tf_layernorm_bwd_partial_bytes(rows, d)) return TF_EWORKSPACE;
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == TF_F16)
+    return ln_bwd_launch<f16>(st, rows, d, dy, lddy, x, ldx, gamma, mean, rstd, dx, lddx, dgamma, dbeta, partial);
+  if (dtype == TF_BF16)
+    return ln_bwd_launch<bf16>(st, rows, d, dy, lddy, x, ldx, gamma, mean, rstd, dx, lddx, dgamma, dbeta, partial);
+  return TF_EDTYPE;
+}
+
+extern "C" int tf_softmax_fwd(void* stream, int dtype, int64_t rows, int64_t cols, const void* x, int64_t ldx,
+                              void* y, int64_t ldy) {
+  if (!x || !y) return TF_EINVAL;
+  if (bad_rows(rows, cols, ldx) || ldy < cols) return TF_EINVAL;
+  if (rows == 0) return TF_OK;
+  hipStream_t st = (hipStream_t)stream;
+  switch (dtype) {
+    case TF_F16: return softmax_fwd_launch<f16>(st, rows, cols, x, ldx, y, ldy);
+    case TF_BF16: return softmax_fwd_launch<bf16>(st, rows, cols, x, ldx, y, ldy);
+    case TF_F32: return softmax_fwd_launch<float>(st, rows, cols, x, ldx, y, ldy);
+  }
+  return TF_EDTYPE;
+}
+
+extern "C" int tf_softmax_bwd(void* stream, int dtype, int64_t rows, int64_t cols, const void* dy, int64_t lddy,
+                              const void* y, int64_t ldy, void* dx, int64_t lddx) {
+  if (!dy || !y || !dx) return TF_EINVAL;
+  if (bad_rows(rows, cols, ldy) || lddy < cols || lddx < cols) return TF_EINVAL;
+  if (rows == 0) return TF_OK;
+  hipStream_t st = (hipStream_t)stream;
+  switch (dtype) {
+    case TF_F16: return softmax_bwd_launch<f16>(st, rows, cols, dy, lddy, y, ldy, dx, lddx);
+    case TF_BF16: return softmax_bwd_launch<bf16>(st, rows, cols, dy, lddy, y, ldy, dx, lddx);
+    case TF_F32: return softmax_bwd_launch<float>(st, rows, cols, dy, lddy, y, ldy, dx, lddx);
+  }
+  return TF_EDTYPE;
+}

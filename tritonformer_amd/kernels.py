@@ -1,0 +1,311 @@
+"""Launcher functions: torch tensors in, one C-ABI call each, torch tensors out.
+
+They take the place of the launchers under the reference's
+``tritonformer/kernels/`` (``mm``/``gemm``/``bmm``, ``flash_wrapper_*``,
+``layernorm_fwd``/``dx_layernorm``/``layernorm_da_db``, ``softmax_*``,
+``cross_entropy_*``, ``unbroadcast_leading``, ``mask_grad``).  Outputs and
+scratch buffers are ``torch.empty`` tensors owned by the caller's allocator;
+the native side keeps nothing.
+"""
+import math
+from functools import lru_cache
+
+import torch
+
+from . import _lib
+from ._lib import KMAJOR, KMINOR, check, dtype_code, load, require_cuda, stream_ptr
+
+
+def _rows2d(x):
+    """View x as (rows, last) with a single row stride; copy only if needed."""
+    if x.stride(-1) != 1 or not x.is_contiguous():
+        x = x.contiguous()
+    return x, x.numel() // x.shape[-1], x.shape[-1]
+
+
+@lru_cache(maxsize=None)
+def _gemm_ws(la, lb, m, n, k):
+    return load().tf_gemm_workspace_bytes(la, lb, m, n, k)
+
+
+def _gemm(dtype, la, lb, m, n, k, a, lda, b, ldb, c, ldc, bias, relu):
+    lib = load()
+    ws_bytes = _gemm_ws(la, lb, m, n, k)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=c.device) if ws_bytes else None
+    check(lib.tf_gemm(stream_ptr(), dtype_code(dtype), la, lb, m, n, k, a.data_ptr(), lda, b.data_ptr(), ldb,
+                      c.data_ptr(), ldc, bias.data_ptr() if bias is not None else None, int(relu),
+                      ws.data_ptr() if ws is not None else None, ws_bytes))
+
+
+def _check_linear(a, b, bias=None):
+    # same preconditions as kernels/gemm.py:370-377, 584-591 of the reference
+    if a.ndim != 3 or b.ndim != 2:
+        raise ValueError("Incorrect number of dimensions for LHS or RHS")
+    if a.shape[2] != b.shape[0]:
+        raise ValueError("Inner dimensions of the two operands do not match")
+    if a.dtype != b.dtype or (bias is not None and bias.dtype != a.dtype):
+        raise TypeError("operands must share one 16-bit dtype")
+    if bias is not None and (bias.ndim != 1 or bias.shape[0] != b.shape[1]):
+        raise ValueError("bias must have one entry per output column")
+    require_cuda(a, b, bias)
+
+
+def gemm(a, b, bias=None, fuse_relu=False):
+    """``relu?(a @ b + bias)`` for a (B, S, in), b (in, out) — reference ``mm``
+    (kernels/gemm.py:361-401) and ``gemm`` (kernels/gemm.py:572-616)."""
+    _check_linear(a, b, bias)
+    a2, m, k = _rows2d(a)
+    n = b.shape[1]
+    if b.stride(-1) == 1 and b.stride(0) >= n:
+        lb, ldb = KMINOR, b.stride(0)          # (in, out) row-major: contraction strided
+    elif b.stride(0) == 1 and b.stride(1) >= k:
+        lb, ldb = KMAJOR, b.stride(1)          # a transposed view, as linear.py:23 passes
+    else:
+        b = b.contiguous()
+        lb, ldb = KMINOR, n
+    if bias is not None and not bias.is_contiguous():
+        bias = bias.contiguous()
+    out = torch.empty(a.shape[:-1] + (n,), dtype=a.dtype, device=a.device)
+    _gemm(a.dtype, KMAJOR, lb, m, n, k, a2, k, b, ldb, out, n, bias, fuse_relu)
+    return out
+
+
+def mm(a, b, fuse_relu=False):
+    return gemm(a, b, None, fuse_relu)
+
+
+def mm_dw(x, grad):
+    """``sum_b x[b]^T @ grad[b]`` -> (in, out): reference ``bmm`` of the
+    transposed view (kernels/gemm.py:161-200) followed by ``torch.sum`` over the
+    batch (linear.py:24-25), as ONE contraction over all B*S tokens."""
+    if x.shape[:-1] != grad.shape[:-1]:
+        raise ValueError("Leading dimensions of the two operands do not match")
+    if x.dtype != grad.dtype:
+        raise TypeError("operands must share one 16-bit dtype")
+    require_cuda(x, grad)
+    x2, t, kin = _rows2d(x)
+    g2, _, nout = _rows2d(grad)
+    out = torch.empty((kin, nout), dtype=x.dtype, device=x.device)
+    _gemm(x.dtype, KMINOR, KMINOR, kin, nout, t, x2, kin, g2, nout, out, nout, None, False)
+    return out
+
+
+def unbroadcast_leading(x):
+    """Sum over every dimension but the last, fp32 accumulation -> (cols,)
+    (reference kernels/reductions.py:97-122)."""
+    require_cuda(x)
+    lib = load()
+    x2, rows, cols = _rows2d(x)
+    out = torch.empty((cols,), dtype=x.dtype, device=x.device)
+    pb = lib.tf_colsum_partial_bytes(rows, cols)
+    part = torch.empty(pb, dtype=torch.uint8, device=x.device)
+    check(lib.tf_colsum(stream_ptr(), dtype_code(x.dtype), rows, cols, x2.data_ptr(), cols, out.data_ptr(),
+                        part.data_ptr(), pb))
+    return out
+
+
+def mask_grad(grad, out_act):
+    """``where(out_act > 0, grad, 0)`` into a NEW tensor (the reference,
+    kernels/activation.py:27-44, overwrites ``grad``)."""
+    require_cuda(grad, out_act)
+    if grad.shape != out_act.shape or grad.dtype != out_act.dtype:
+        raise ValueError("grad and activation must agree in shape and dtype")
+    g2, rows, cols = _rows2d(grad)
+    a2, _, _ = _rows2d(out_act)
+    out = torch.empty(grad.shape, dtype=grad.dtype, device=grad.device)
+    check(load().tf_relu_mask(stream_ptr(), dtype_code(grad.dtype), rows, cols, g2.data_ptr(), cols, a2.data_ptr(),
+                              cols, out.data_ptr(), cols))
+    return out
+
+
+# --------------------------------------------------------------------------- attention
+def _attn_layout(q, *others):
+    """All tensors must share q's strides, unit stride along hd and 16-byte
+    aligned rows; otherwise everything is copied to contiguous (B, nh, S, hd)."""
+    ok = q.stride(-1) == 1 and all(s % 8 == 0 for s in q.stride()[:-1]) and q.data_ptr() % 16 == 0
+    ok = ok and all(t.stride() == q.stride() and t.data_ptr() % 16 == 0 for t in others)
+    if ok:
+        return (q,) + tuple(others)
+    return tuple(t.contiguous() for t in (q,) + tuple(others))
+
+
+def _check_attn(q, k, v, bias):
+    if q.ndim != 4 or q.shape != k.shape or q.shape != v.shape:
+        raise ValueError("q, k, v must be (B, nh, S, hd) tensors of one shape")
+    b, nh, s, hd = q.shape
+    if hd not in (32, 64, 128):
+        raise ValueError("Only head_dims of [32,64,128] are supported.")
+    if s % 64 != 0:
+        raise ValueError("Sequence length must be a multiple of the 64-row block size")
+    if not (q.dtype == k.dtype == v.dtype) or q.dtype not in (torch.float16, torch.bfloat16):
+        raise TypeError("q, k, v must share one 16-bit dtype")
+    require_cuda(q, k, v, bias)
+    if bias is not None:
+        # kernels/biased_attention.py:199-207 of the reference
+        if bias.ndim != 3 or bias.shape[0] != nh:
+            raise ValueError("attention bias must be (nh, S', S')")
+        if bias.shape[1] != bias.shape[2] or bias.shape[1] < s:
+            raise ValueError("attention bias must be square and cover the sequence")
+        if bias.dtype != q.dtype:
+            raise TypeError("attention bias must have the dtype of q")
+
+
+def _bias_args(bias):
+    if bias is None:
+        return None, None, 0, 0
+    if bias.stride(-1) != 1 or bias.stride(0) % 4 or bias.stride(1) % 4 or bias.data_ptr() % 8:
+        bias = bias.contiguous()
+    return bias, bias.data_ptr(), bias.stride(0), bias.stride(1)
+
+
+def flash_wrapper_fwd(q, k, v, bias=None):
+    """Causal attention forward -> (out, lse).  ``out`` has q's strides; ``lse``
+    is (B, nh, S) fp32 in the log2 domain (the reference keeps fp16 m and l,
+    kernels/attention.py:171-217 and kernels/biased_attention.py:188-245)."""
+    _check_attn(q, k, v, bias)
+    q, k, v = _attn_layout(q, k, v)
+    b, nh, s, hd = q.shape
+    out = torch.empty_like(q)
+    if out.stride() != q.stride():
+        out = torch.empty_strided(q.shape, q.stride(), dtype=q.dtype, device=q.device)
+    lse = torch.empty((b, nh, s), dtype=torch.float32, device=q.device)
+    bias, bptr, bsh, bsr = _bias_args(bias)
+    check(load().tf_attn_fwd(stream_ptr(), dtype_code(q.dtype), b, nh, s, hd, q.data_ptr(), k.data_ptr(),
+                             v.data_ptr(), out.data_ptr(), q.stride(0), q.stride(1), q.stride(2), lse.data_ptr(),
+                             bptr, bsh, bsr, 1.0 / math.sqrt(hd)))
+    return out, lse
+
+
+def flash_wrapper_bwd(grad_out, out, q, k, v, lse, bias=None):
+    """Causal attention backward -> (dq, dk, dv), each with q's strides
+    (reference kernels/attention.py:550-607, kernels/biased_attention.py:598-660)."""
+    _check_attn(q, k, v, bias)
+    q, k, v, out = _attn_layout(q, k, v, out)
+    if grad_out.stride() != q.stride() or grad_out.data_ptr() % 16:
+        g = torch.empty_strided(q.shape, q.stride(), dtype=q.dtype, device=q.device)
+        g.copy_(grad_out)
+        grad_out = g
+    b, nh, s, hd = q.shape
+    dq = torch.empty_strided(q.shape, q.stride(), dtype=q.dtype, device=q.device)
+    dk = torch.empty_strided(q.shape, q.stride(), dtype=q.dtype, device=q.device)
+    dv = torch.empty_strided(q.shape, q.stride(), dtype=q.dtype, device=q.device)
+    delta = torch.empty((b, nh, s), dtype=torch.float32, device=q.device)
+    bias, bptr, bsh, bsr = _bias_args(bias)
+    check(load().tf_attn_bwd(stream_ptr(), dtype_code(q.dtype), b, nh, s, hd, q.data_ptr(), k.data_ptr(),
+                             v.data_ptr(), out.data_ptr(), grad_out.data_ptr(), dq.data_ptr(), dk.data_ptr(),
+                             dv.data_ptr(), q.stride(0), q.stride(1), q.stride(2), lse.data_ptr(),
+                             delta.data_ptr(), bptr, bsh, bsr, 1.0 / math.sqrt(hd)))
+    return dq, dk, dv
+
+
+def flash_wrapper_fwd_attn_bias(q, k, v, attn_bias):
+    return flash_wrapper_fwd(q, k, v, attn_bias)
+
+
+def flash_wrapper_bwd_attn_bias(grad_out, out, q, k, v, lse, attn_bias):
+    return flash_wrapper_bwd(grad_out, out, q, k, v, lse, attn_bias)
+
+
+# --------------------------------------------------------------------------- layernorm
+def _check_ln(x, d):
+    # kernels/layernorm.py:68-71 of the reference: 3-D, 16-bit, on the GPU
+    if x.ndim != 3:
+        raise ValueError("LayerNorm input must be 3-dimensional (B, S, d)")
+    if x.dtype not in (torch.float16, torch.bfloat16):
+        raise TypeError("LayerNorm input must be float16 or bfloat16")
+    if x.shape[-1] != d:
+        raise ValueError("LayerNorm parameters do not match the last dimension")
+    require_cuda(x)
+
+
+def layernorm_fwd(x, alpha, beta, eps):
+    """-> (y, mean, rstd); reference kernels/layernorm.py:64-87."""
+    _check_ln(x, alpha.shape[0])
+    if alpha.dtype != x.dtype or beta.dtype != x.dtype:
+        raise TypeError("LayerNorm parameters must have the input's dtype")
+    x2, rows, d = _rows2d(x)
+    y = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    mean = torch.empty((rows,), dtype=torch.float32, device=x.device)
+    rstd = torch.empty((rows,), dtype=torch.float32, device=x.device)
+    check(load().tf_layernorm_fwd(stream_ptr(), dtype_code(x.dtype), rows, d, x2.data_ptr(), d,
+                                  alpha.contiguous().data_ptr(), beta.contiguous().data_ptr(), float(eps),
+                                  y.data_ptr(), d, mean.data_ptr(), rstd.data_ptr()))
+    return y, mean, rstd
+
+
+def layernorm_bwd(grad_out, x, alpha, mean, rstd):
+    """-> (dx, dalpha, dbeta); reference dx_layernorm (kernels/layernorm.py:140-162)
+    and layernorm_da_db (kernels/layernorm.py:226-259) in one pass."""
+    lib = load()
+    x2, rows, d = _rows2d(x)
+    g2, _, _ = _rows2d(grad_out)
+    dx = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    da = torch.empty((d,), dtype=x.dtype, device=x.device)
+    db = torch.empty((d,), dtype=x.dtype, device=x.device)
+    pb = lib.tf_layernorm_bwd_partial_bytes(rows, d)
+    part = torch.empty(pb, dtype=torch.uint8, device=x.device)
+    check(lib.tf_layernorm_bwd(stream_ptr(), dtype_code(x.dtype), rows, d, g2.data_ptr(), d, x2.data_ptr(), d,
+                               alpha.contiguous().data_ptr(), mean.data_ptr(), rstd.data_ptr(), dx.data_ptr(), d,
+                               da.data_ptr(), db.data_ptr(), part.data_ptr(), pb))
+    return dx, da, db
+
+
+# --------------------------------------------------------------------------- softmax
+def softmax_fwd(x):
+    """Row softmax over the last dim (reference kernels/softmax.py:37-54)."""
+    require_cuda(x)
+    if x.ndim != 3:
+        raise ValueError("Softmax input must be 3-dimensional")
+    x2, rows, cols = _rows2d(x)
+    y = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    check(load().tf_softmax_fwd(stream_ptr(), dtype_code(x.dtype), rows, cols, x2.data_ptr(), cols, y.data_ptr(),
+                                cols))
+    return y
+
+
+def softmax_bwd(grad_out, saved_out):
+    """``y * (dy - sum(y*dy))`` into a new tensor (reference kernels/softmax.py:95-111
+    writes over grad_out)."""
+    require_cuda(grad_out, saved_out)
+    g2, rows, cols = _rows2d(grad_out)
+    y2, _, _ = _rows2d(saved_out)
+    dx = torch.empty(saved_out.shape, dtype=saved_out.dtype, device=saved_out.device)
+    check(load().tf_softmax_bwd(stream_ptr(), dtype_code(saved_out.dtype), rows, cols, g2.data_ptr(), cols,
+                                y2.data_ptr(), cols, dx.data_ptr(), cols))
+    return dx
+
+
+# --------------------------------------------------------------------------- cross entropy
+def cross_entropy_fwd(logits, labels):
+    """-> (per-row loss in logits' dtype, lse fp32); reference
+    kernels/crossentropy.py:47-75 (which keeps the full (N, V) matrix instead)."""
+    if logits.ndim != 2 or labels.ndim != 1 or labels.shape[0] != logits.shape[0]:
+        raise ValueError("cross entropy takes (N, V) logits and (N,) labels")
+    if labels.dtype != torch.int64:
+        raise TypeError("labels must be int64")
+    if logits.dtype not in (torch.float16, torch.bfloat16):
+        raise TypeError("logits must be float16 or bfloat16")
+    require_cuda(logits, labels)
+    if logits.stride(-1) != 1:
+        logits = logits.contiguous()
+    labels = labels.contiguous()
+    n, v = logits.shape
+    loss = torch.empty((n,), dtype=logits.dtype, device=logits.device)
+    lse = torch.empty((n,), dtype=torch.float32, device=logits.device)
+    check(load().tf_cross_entropy_fwd(stream_ptr(), dtype_code(logits.dtype), n, v, logits.data_ptr(),
+                                      logits.stride(0), labels.data_ptr(), loss.data_ptr(), lse.data_ptr()))
+    return loss, lse, logits, labels
+
+
+def cross_entropy_bwd(grad_out, logits, labels, lse):
+    """``(softmax(logits) - onehot) * grad_out[:, None]`` (reference
+    kernels/crossentropy.py:110-127 and the multiply at crossentropy.py:24)."""
+    n, v = logits.shape
+    if grad_out.dtype != logits.dtype:
+        grad_out = grad_out.to(logits.dtype)
+    gstride = grad_out.stride(0) if grad_out.ndim == 1 else 0
+    dlogits = torch.empty((n, v), dtype=logits.dtype, device=logits.device)
+    check(load().tf_cross_entropy_bwd(stream_ptr(), dtype_code(logits.dtype), n, v, logits.data_ptr(),
+                                      logits.stride(0), labels.data_ptr(), lse.data_ptr(), grad_out.data_ptr(),
+                                      gstride, dlogits.data_ptr(), v))
+    return dlogits

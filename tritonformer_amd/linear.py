@@ -1,0 +1,88 @@
+"""Linear-layer autograd Functions; same classes and ``apply`` signatures as
+the reference's tritonformer/linear.py.  Weight layout is (in, out): y = x @ W."""
+import torch
+from torch.autograd import Function
+
+from ._amp import amp_bwd, amp_fwd
+from .kernels import gemm, mask_grad, mm, mm_dw, unbroadcast_leading
+
+
+def _grads(ctx, grad_output, inputs, weights):
+    """dX = dY W^T (W read as stored, contraction along its rows) and
+    dW = X^T dY with the batch folded into the contraction
+    (reference linear.py:21-25 goes through bmm + torch.sum)."""
+    grad_input = mm(grad_output, weights.T) if ctx.needs_input_grad[0] else None
+    grad_weights = mm_dw(inputs, grad_output) if ctx.needs_input_grad[1] else None
+    return grad_input, grad_weights
+
+
+class LinearNoBias(Function):
+    """MM(X,A) kernel call (reference linear.py:10-25)."""
+
+    @staticmethod
+    @amp_fwd
+    def forward(ctx, input, weight):
+        ctx.save_for_backward(input, weight)
+        return mm(input, weight)
+
+    @staticmethod
+    @amp_bwd
+    def backward(ctx, grad_output):
+        inputs, weights = ctx.saved_tensors
+        return _grads(ctx, grad_output, inputs, weights)
+
+
+class LinearBias(Function):
+    """Fused GEMM(X,A,B) in a single kernel call (reference linear.py:28-44)."""
+
+    @staticmethod
+    @amp_fwd
+    def forward(ctx, input, weight, bias):
+        ctx.save_for_backward(input, weight)
+        return gemm(input, weight, bias, False)
+
+    @staticmethod
+    @amp_bwd
+    def backward(ctx, grad_output):
+        inputs, weights = ctx.saved_tensors
+        grad_input, grad_weights = _grads(ctx, grad_output, inputs, weights)
+        grad_bias = unbroadcast_leading(grad_output) if ctx.needs_input_grad[2] else None
+        return grad_input, grad_weights, grad_bias
+
+
+class LinearNoBiasReLU(Function):
+    """Fused ReLU(MM(X,A)) in a single kernel call (reference linear.py:47-69)."""
+
+    @staticmethod
+    @amp_fwd
+    def forward(ctx, input, weight):
+        out_w_act = mm(input, weight, True)
+        ctx.save_for_backward(input, weight, out_w_act)
+        return out_w_act
+
+    @staticmethod
+    @amp_bwd
+    def backward(ctx, grad_output):
+        inputs, weights, out_w_act = ctx.saved_tensors
+        grad_output = mask_grad(grad_output, out_w_act)  # new tensor: autograd's buffer stays intact
+        return _grads(ctx, grad_output, inputs, weights)
+
+
+class LinearBiasReLU(Function):
+    """Fused ReLU(GEMM(X,A,bias)) in a single kernel call (reference linear.py:72-102)."""
+
+    @staticmethod
+    @amp_fwd
+    def forward(ctx, input, weight, bias):
+        out_w_act = gemm(input, weight, bias, True)
+        ctx.save_for_backward(input, weight, out_w_act)
+        return out_w_act
+
+    @staticmethod
+    @amp_bwd
+    def backward(ctx, grad_output):
+        inputs, weights, out_w_act = ctx.saved_tensors
+        grad_output = mask_grad(grad_output, out_w_act)
+        grad_input, grad_weights = _grads(ctx, grad_output, inputs, weights)
+        grad_bias = unbroadcast_leading(grad_output) if ctx.needs_input_grad[2] else None
+        return grad_input, grad_weights, grad_bias
