@@ -1,0 +1,226 @@
+#!/usr/bin/env python3
+"""Headline benchmark: one fwd+bwd training step of the 410M / ctx 2048 / bs 4
+GPT-2 style decoder (24 layers, d=1024, 16 heads x 64, MLP 4096 ReLU, no linear
+bias, no ALiBi, vocab 50304) on ONE MI355X, fp16 autocast over fp32 master
+weights, every Linear / LayerNorm / attention / cross-entropy running on the
+tritonformer_amd HIP kernels.  Prints one JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
+
+value        = algorithmic FLOPs of the step (6*T*P_mat + 7*L*B*S^2*d) / step time, in TFLOP/s
+roofline     = the GEMM kernel (dominant in time): algorithmic FLOPs per launch / mean launch
+               duration, the duration measured with HIP events recorded on the launch stream
+               around every GEMM launch in instrumented repeats of the same steps
+cpu_baseline = the fp32 PyTorch oracle (oracle/ref_torch.py) on the host cores, on a bounded
+               sample: the same step with the stack cut to 2 layers
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA
+PEAK_HBM_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (layers, d, heads, head_dim, ffn, seq, batch, linear_bias, alibi)
+    "gpt2-410m-ctx2048-bs4": (24, 1024, 16, 64, 4096, 2048, 4, False, False),
+    "gpt2-160m-ctx2048-bs8": (12, 768, 12, 64, 3072, 2048, 8, True, False),
+    "gpt2-840m-alibi-ctx4096-bs1": (24, 1536, 24, 64, 6144, 4096, 1, False, True),
+    "gpt2-1.4b-ctx2048-bs2": (24, 2048, 16, 128, 8192, 2048, 2, False, False),
+    "gpt2-tiny-ctx256-bs2": (4, 256, 4, 64, 1024, 256, 2, True, False),
+}
+VOCAB = 50304
+
+
+def step_flops(L, d, f, S, B):
+    p_mat = L * (4 * d * d + 2 * d * f) + d * VOCAB
+    return 6.0 * B * S * p_mat + 7.0 * L * B * S * S * d
+
+
+def gemm_flops(L, d, f, S, B):
+    return 6.0 * B * S * (L * (4 * d * d + 2 * d * f) + d * VOCAB)
+
+
+def make_model(name, device, dtype):
+    from tritonformer_amd.transformer import Transformer, TransformerConfig
+
+    L, d, nh, hd, f, S, B, lin_bias, alibi = WORKLOADS[name]
+    cfg = TransformerConfig(VOCAB, d, S, nh, hd, f, L, lin_bias, alibi)
+    torch.manual_seed(0)
+    model = Transformer(cfg, device=device, param_dtype=torch.float32)
+    model.logits_out.weight.data.normal_(0.0, 0.02)  # reference init zeros the LM head; keep the loss path live
+    tokens = torch.randint(0, VOCAB, (B, S), device=device)
+    return model, tokens
+
+
+def run_steps(model, tokens, n, dtype):
+    loss = None
+    for _ in range(n):
+        model.zero_grad(set_to_none=True)
+        with torch.autocast("cuda", dtype=dtype):
+            _, loss = model(tokens, tokens)
+        loss.backward()
+    return loss
+
+
+class GemmTimer:
+    """HIP events on the current (launch) stream around every tf_gemm call."""
+
+    def __init__(self):
+        self.records = []
+
+    def __enter__(self):
+        from tritonformer_amd import kernels
+
+        self._kernels = kernels
+        self._orig = kernels._gemm
+
+        def timed(dtype, la, lb, m, n, k, *rest):
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record()
+            self._orig(dtype, la, lb, m, n, k, *rest)
+            e1.record()
+            self.records.append(((la, lb, m, n, k), e0, e1))
+
+        kernels._gemm = timed
+        return self
+
+    def __exit__(self, *exc):
+        self._kernels._gemm = self._orig
+        torch.cuda.synchronize()
+        self.by_shape = {}
+        for key, e0, e1 in self.records:
+            ms = e0.elapsed_time(e1)
+            cnt, tot = self.by_shape.get(key, (0, 0.0))
+            self.by_shape[key] = (cnt + 1, tot + ms)
+        return False
+
+
+def cpu_baseline(name, seconds_cap=60.0):
+    """fp32 oracle on the host: same B, S, d, heads, ffn, vocab; depth cut to 2 layers."""
+    from oracle import ref_torch as R
+
+    L, d, nh, hd, f, S, B, lin_bias, alibi = WORKLOADS[name]
+    Ls = min(L, 2)
+    cores = int(os.environ.get("OMP_NUM_THREADS", 0)) or os.cpu_count()
+    cores = min(cores, os.cpu_count())
+    torch.set_num_threads(cores)
+    cfg = R.RefConfig(VOCAB, d, S, nh, hd, f, Ls, lin_bias, alibi)
+    torch.manual_seed(0)
+    model = R.RefTransformer(cfg, sdpa=True)
+    model.logits_out.weight.data.normal_(0.0, 0.02)
+    tokens = torch.randint(0, VOCAB, (B, S))
+    flops = step_flops(Ls, d, f, S, B)
+    times = []
+    t_begin = time.perf_counter()
+    for i in range(3):  # first pass is the warm-up
+        model.zero_grad(set_to_none=True)
+        t0 = time.perf_counter()
+        _, loss = model(tokens, tokens)
+        loss.backward()
+        times.append(time.perf_counter() - t0)
+        if time.perf_counter() - t_begin > seconds_cap:
+            break
+    best = min(times[1:]) if len(times) > 1 else times[0]
+    return {
+        "value": round(flops / best / 1e12, 4),
+        "unit": "TFLOP/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"fp32 PyTorch oracle, same step with the stack cut to {Ls} of {L} layers "
+                  f"(B={B}, S={S}, d={d}, vocab={VOCAB}; {flops / 1e12:.2f} TFLOP), best of {max(len(times) - 1, 1)} "
+                  f"after 1 warm-up, {best:.2f} s/step",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="gpt2-410m-ctx2048-bs4", choices=sorted(WORKLOADS))
+    ap.add_argument("--dtype", default="fp16", choices=["fp16", "bf16"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-roofline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported "
+                 "(no collectives are part of it)")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: needs an MI355X (no CPU path exists for the kernels)")
+
+    dtype = torch.float16 if args.dtype == "fp16" else torch.bfloat16
+    device = torch.device("cuda:0")
+    L, d, nh, hd, f, S, B, lin_bias, alibi = WORKLOADS[args.workload]
+    model, tokens = make_model(args.workload, device, dtype)
+
+    run_steps(model, tokens, args.warmup, dtype)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    loss = run_steps(model, tokens, args.steps, dtype)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms = elapsed / args.steps * 1e3
+    flops = step_flops(L, d, f, S, B)
+    tflops = flops / (ms * 1e-3) / 1e12
+
+    out = {
+        "metric": "fwd+bwd model TFLOPs on 1 MI355X, 410M ctx2048 bs4; % of fp16 MFMA peak",
+        "value": round(tflops, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms, 3),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": args.dtype,
+        "data": "synthetic",
+        "config": {"workload": args.workload, "layers": L, "d_model": d, "heads": nh, "head_dim": hd, "ffn": f,
+                   "seq_len": S, "global_batch": B, "vocab": VOCAB, "linear_bias": lin_bias, "alibi": alibi,
+                   "master_weights": "fp32", "autocast": args.dtype, "parallelism": "single GPU"},
+        "pct_of_fp16_mfma_peak": round(100.0 * tflops / PEAK_FP16_TFLOPS, 2),
+        "tokens_per_s": round(B * S / (ms * 1e-3), 1),
+        "step_tflop": round(flops / 1e12, 3),
+        "loss": round(float(loss), 4),
+    }
+
+    if not args.no_roofline:
+        reps = max(1, min(args.steps, 5))
+        with GemmTimer() as gt:
+            run_steps(model, tokens, reps, dtype)
+        launches = sum(c for c, _ in gt.by_shape.values())
+        total_ms = sum(t for _, t in gt.by_shape.values())
+        gflops = gemm_flops(L, d, f, S, B) * reps
+        achieved = gflops / (total_ms * 1e-3) / 1e12
+        out["roofline"] = {
+            "bound": "mfma",
+            "kernel": "tfa::gemm_kernel (all instantiations; fwd X.W, dX = dY.W^T, dW = X^T.dY)",
+            "achieved": round(achieved, 2),
+            "peak": PEAK_FP16_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(achieved / PEAK_FP16_TFLOPS, 4),
+            "traffic": None,
+            "launches_per_step": launches // reps,
+            "flop_per_launch": round(gflops / launches, 1),
+            "avg_launch_us": round(total_ms / launches * 1e3, 2),
+            "gemm_ms_per_step": round(total_ms / reps, 3),
+            "measured": f"HIP events on the launch stream around each tf_gemm call, {reps} instrumented steps "
+                        "run after the timed ones (split-contraction launches include their reduce kernel)",
+        }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(args.workload)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

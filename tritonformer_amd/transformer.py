@@ -1,0 +1,193 @@
+"""GPT-2 style decoder built on the tritonformer_amd operators.
+
+Host-side counterpart of the reference's top-level ``transformer.py``: the same
+``TransformerConfig`` fields, module tree and parameter names
+(``embed_tokens``, ``embed_positions``, ``layer_list.{i}.input_layernorm``,
+``...attention.{q,k,v,out}_proj``, ``...mlp.dense_h_to_4h`` / ``dense_4h_to_h``,
+``final_layernorm``, ``logits_out``, buffer ``attn_bias``), the same
+initialisation and the same loss (mean over the B*(S-1) shifted positions), so
+a state dict moves between the two unchanged.  Two additions: the device is a
+parameter instead of the hard-coded "cuda:0", and ``param_dtype`` selects fp16
+parameters (the reference's choice, transformer.py:124-151) or fp32 master
+weights used under autocast.
+"""
+import math
+from dataclasses import dataclass
+from typing import List, Optional, Tuple
+
+import torch
+import torch.nn as nn
+
+from . import cross_entropy_loss, fast_causal_attention, fast_causal_attention_with_bias
+from . import nn as tnn
+
+
+@dataclass(frozen=True)
+class TransformerConfig:
+    vocab_size: int
+    hidden_size: int
+    max_position_embeddings: int
+    num_attention_heads: int
+    head_dim: int
+    ffn_dim: int
+    num_hidden_layers: int
+    use_linear_bias: bool
+    attn_bias: bool
+
+
+def get_slopes(n: int) -> List[float]:
+    """ALiBi slopes (reference transformer.py:37-52): for n = 2^k the geometric
+    sequence 2^(-8/n), 2^(-16/n), ...; otherwise the slopes of the largest
+    power of two below n followed by every other slope of the next power."""
+    def power_of_two(m):
+        base = 2.0 ** (-(2.0 ** -(math.log2(m) - 3)))
+        return [base ** (i + 1) for i in range(m)]
+
+    if n & (n - 1) == 0:
+        return power_of_two(n)
+    lower = 1 << (n.bit_length() - 1)
+    return power_of_two(lower) + get_slopes(2 * lower)[0::2][: n - lower]
+
+
+def generate_alibi_mask(seq_len: int, num_heads: int, device=None, dtype=torch.float16) -> torch.Tensor:
+    """(1, nh, S, S) additive bias: -slope_h * (i - j) for j <= i, -inf above
+    the diagonal, with distances, slopes and their product all rounded to
+    ``dtype`` as in reference transformer.py:55-75."""
+    pos = torch.arange(seq_len, device=device)
+    dist = (pos[None, :] - pos[:, None]).clamp(max=0).to(dtype)            # -(i - j) on and below the diagonal
+    slopes = torch.tensor(get_slopes(num_heads), device=device, dtype=dtype)
+    bias = dist[None] * slopes[:, None, None]
+    above = pos[None, :] > pos[:, None]
+    return bias.masked_fill(above[None], float("-inf"))[None]
+
+
+def _weights_init(model: nn.Module, num_layers: int) -> None:
+    """Reference transformer.py:83-105: N(0, 0.02) for every Linear/Embedding
+    weight, N(0, 0.02/sqrt(2L)) for the two residual-output projections, zeros
+    for the LM head and all biases, LayerNorm gamma=1 beta=0."""
+    for name, m in model.named_modules():
+        if isinstance(m, tnn.Linear):
+            std = 0.02
+            leaf = name.rsplit(".", 1)[-1]
+            if leaf in ("out_proj", "dense_4h_to_h"):
+                std = 0.02 / math.sqrt(2 * num_layers)
+            if leaf == "logits_out":
+                m.weight.data.zero_()
+            else:
+                m.weight.data.normal_(mean=0.0, std=std)
+            if m.bias is not None:
+                nn.init.zeros_(m.bias)
+        elif isinstance(m, nn.Embedding):
+            m.weight.data.normal_(mean=0.0, std=0.02)
+        elif isinstance(m, tnn.LayerNorm):
+            nn.init.ones_(m.weight)
+            nn.init.zeros_(m.bias)
+
+
+class CausalAttention(nn.Module):
+    """Self-attention block (reference transformer.py:113-190)."""
+
+    def __init__(self, config: TransformerConfig, device=None, dtype=torch.float16):
+        super().__init__()
+        self.hidden_size = config.hidden_size
+        self.num_attention_heads = config.num_attention_heads
+        self.hidden_size_per_attention_head = config.hidden_size // config.num_attention_heads
+        kw = dict(device=device, dtype=dtype, bias=False)
+        self.q_proj = tnn.Linear(config.hidden_size, config.hidden_size, **kw)
+        self.k_proj = tnn.Linear(config.hidden_size, config.hidden_size, **kw)
+        self.v_proj = tnn.Linear(config.hidden_size, config.hidden_size, **kw)
+        self.out_proj = tnn.Linear(config.hidden_size, config.hidden_size, **kw)
+
+    def _heads(self, x: torch.Tensor) -> torch.Tensor:
+        b, s, _ = x.shape  # "b s (nh hd) -> b nh s hd" as a view, strides (S*d, hd, d, 1)
+        return x.view(b, s, self.num_attention_heads, self.hidden_size_per_attention_head).permute(0, 2, 1, 3)
+
+    def forward(self, hidden_states: torch.Tensor, attn_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+        batch_size, q_seq_len, hidden_dim = hidden_states.shape
+        query_layer = self._heads(self.q_proj(hidden_states))
+        key_layer = self._heads(self.k_proj(hidden_states))
+        value_layer = self._heads(self.v_proj(hidden_states))
+        if attn_bias is None:
+            attn = fast_causal_attention.apply(query_layer, key_layer, value_layer)
+        else:
+            attn = fast_causal_attention_with_bias.apply(query_layer, key_layer, value_layer, attn_bias)
+        # attn keeps q's strides, so this is a view, not a copy
+        context_layer = attn.transpose(1, 2).contiguous().view(batch_size, q_seq_len, hidden_dim)
+        return self.out_proj(context_layer)
+
+
+class MLPBlock(nn.Module):
+    """Linear(+bias)+ReLU fused, then Linear(+bias) (reference transformer.py:193-217)."""
+
+    def __init__(self, config: TransformerConfig, device=None, dtype=torch.float16):
+        super().__init__()
+        self.dense_h_to_4h = tnn.Linear(config.hidden_size, config.ffn_dim, device=device, dtype=dtype,
+                                        fuse_activation=True, bias=config.use_linear_bias)
+        self.dense_4h_to_h = tnn.Linear(config.ffn_dim, config.hidden_size, device=device, dtype=dtype,
+                                        bias=config.use_linear_bias)
+
+    def forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
+        return self.dense_4h_to_h(self.dense_h_to_4h(hidden_states))
+
+
+class TransformerLayer(nn.Module):
+    """Pre-LN block (reference transformer.py:220-251)."""
+
+    def __init__(self, config: TransformerConfig, device=None, dtype=torch.float16):
+        super().__init__()
+        self.input_layernorm = tnn.LayerNorm(config.hidden_size, device=device, dtype=dtype)
+        self.post_attention_layernorm = tnn.LayerNorm(config.hidden_size, device=device, dtype=dtype)
+        self.attention = CausalAttention(config, device=device, dtype=dtype)
+        self.mlp = MLPBlock(config, device=device, dtype=dtype)
+
+    def forward(self, hidden_states: torch.Tensor, attn_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+        hidden_states = hidden_states + self.attention(self.input_layernorm(hidden_states), attn_bias)
+        return hidden_states + self.mlp(self.post_attention_layernorm(hidden_states))
+
+
+class Transformer(nn.Module):
+    """Decoder stack + LM head + shifted cross-entropy (reference transformer.py:254-346)."""
+
+    def __init__(self, config: TransformerConfig, device=None, param_dtype=torch.float16):
+        super().__init__()
+        self.config = config
+        self.embed_tokens = nn.Embedding(config.vocab_size, config.hidden_size, device=device, dtype=param_dtype)
+        self.embed_positions = None
+        if not config.attn_bias:
+            self.embed_positions = nn.Embedding(config.max_position_embeddings, config.hidden_size, device=device,
+                                                dtype=param_dtype)
+        self.layer_list = nn.ModuleList(
+            [TransformerLayer(config, device=device, dtype=param_dtype) for _ in range(config.num_hidden_layers)]
+        )
+        self.final_layernorm = tnn.LayerNorm(config.hidden_size, device=device, dtype=param_dtype)
+        self.logits_out = tnn.Linear(config.hidden_size, config.vocab_size, bias=False, device=device,
+                                     dtype=param_dtype, fuse_activation=False)
+        _weights_init(self, config.num_hidden_layers)
+        if config.attn_bias:
+            # the bias is an activation-side tensor: always 16-bit, like the reference's
+            self.register_buffer(
+                "attn_bias",
+                generate_alibi_mask(config.max_position_embeddings, config.num_attention_heads, device=device)[0],
+            )
+        else:
+            self.attn_bias = None
+
+    def forward(self, input_ids: torch.Tensor, labels: Optional[torch.Tensor]):
+        batch_size, seq_len = input_ids.shape
+        hidden_states = self.embed_tokens(input_ids)
+        if self.embed_positions is not None:
+            positions = torch.arange(seq_len, device=hidden_states.device)[None].expand(batch_size, -1)
+            hidden_states = hidden_states + self.embed_positions(positions)
+        attn_bias = self.attn_bias
+        if attn_bias is not None and torch.is_autocast_enabled("cuda"):
+            attn_bias = attn_bias.to(torch.get_autocast_dtype("cuda"))
+        for layer in self.layer_list:
+            hidden_states = layer(hidden_states, attn_bias)
+        hidden_states = self.final_layernorm(hidden_states)
+        logits_lm = self.logits_out(hidden_states)
+        if labels is None:
+            return logits_lm
+        shift_logits = logits_lm[..., :-1, :].contiguous()
+        shift_labels = labels[..., 1:].contiguous()
+        loss = cross_entropy_loss.apply(shift_logits.view(-1, shift_logits.size(-1)), shift_labels.view(-1))
+        return logits_lm, loss.mean()
