@@ -71,7 +71,25 @@ int tf_gemm(void* stream, int dtype, int layout_a, int layout_b,
             const void* A, int64_t lda, const void* B, int64_t ldb,
             void* C, int64_t ldc, const void* bias, int relu,
             void* workspace, int64_t workspace_bytes);
+/* As tf_gemm with C stored as `out_dtype`: either `dtype` or TF_F32 (fp32 weight
+ * gradients for fp32 master weights, skipping the separate 16->32 bit cast pass
+ * autograd would otherwise run; the reference keeps fp16 parameters and has no
+ * such case). */
+int tf_gemm_out(void* stream, int dtype, int out_dtype, int layout_a, int layout_b,
+                int64_t M, int64_t N, int64_t K,
+                const void* A, int64_t lda, const void* B, int64_t ldb,
+                void* C, int64_t ldc, const void* bias, int relu,
+                void* workspace, int64_t workspace_bytes);
 int64_t tf_gemm_workspace_bytes(int layout_a, int layout_b, int64_t M, int64_t N, int64_t K);
+/* Diagnostic, no counterpart in the reference (whose Triton autotuner picks
+ * tiles per shape, kernels/gemm.py:15-79): force tile configuration `cfg`
+ * (-1 = automatic) and contraction split `splits` (0 = automatic) for all
+ * later tf_gemm / tf_gemm_workspace_bytes calls of this process. */
+int tf_gemm_tune(int cfg, int splits);
+/* Diagnostic: bit 0 disables the XCD-aware workgroup remap, bit 1 skips the
+ * in-loop operand loads, bit 2 skips the MFMA work (bits 1-2 give WRONG results;
+ * they exist to time the pipeline's parts in isolation). */
+int tf_gemm_debug_flags(int flags);
 
 /* Causal flash attention forward.  q,k,v,o: logical (B, nh, S, hd) with the
  * SAME element strides {sb, sh, ss} and unit stride along hd (the reference

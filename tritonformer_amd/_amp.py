@@ -27,6 +27,8 @@ def amp_fwd(fwd):
     def wrapper(ctx, *args):
         ctx._dtype = torch.get_autocast_dtype("cuda")
         ctx._fwd_used_autocast = False
+        # dtypes the caller passed in, before any autocast cast (fp32 master weights)
+        ctx.arg_dtypes = tuple(a.dtype if isinstance(a, torch.Tensor) else None for a in args)
         if torch.is_autocast_enabled("cuda"):
             dtype = torch.bfloat16 if ctx._dtype == torch.bfloat16 else torch.float16
             with torch.autocast(device_type="cuda", enabled=False):

@@ -36,6 +36,8 @@ struct GemmParams {
   int relu;
   int splits, k_per_split;
   int tiles_m, tiles_n;
+  int flags;  // bit 0: skip the XCD remap (diagnostic)
+  int out_f32;  // C holds fp32 instead of T
 };
 
 // ---------------------------------------------------------------------------
@@ -120,6 +122,70 @@ __device__ __forceinline__ int remap_xcd(int pid, int n) {
   return xcd * q + (xcd < r ? xcd : r) + local;
 }
 
+// Epilogue shared by both kernels: lane holds C[m][n .. n+3] for m = .. + lane%32.
+template <typename T, int TM, int TN, int WTM, int WTN, bool VEC>
+__device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)[TM][TN], int m0, int n0, int wm,
+                                              int wn, int lane, int split) {
+  const T* bias = (const T*)p.bias;
+  T* C = (T*)p.C;
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int m = m0 + wm * WTM + i * 32 + (lane & 31);
+    if (m >= p.M) continue;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int n = n0 + wn * WTN + j * 32 + g * 8 + (lane >> 5) * 4;
+        if (n >= p.N) continue;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = acc[i][j][g * 4 + e];
+        if (p.splits > 1) {
+          float* dst = p.partial + ((int64_t)split * p.M + m) * p.N + n;
+          if (VEC) {
+            f32x4 o = {v[0], v[1], v[2], v[3]};
+            *reinterpret_cast<f32x4*>(dst) = o;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (n + e < p.N) dst[e] = v[e];
+          }
+        } else {
+          if (p.out_f32) {
+            float* Cf = reinterpret_cast<float*>(p.C) + (int64_t)m * p.ldc + n;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              if (n + e < p.N) {
+                const float x = v[e] + (bias ? (float)bias[n + e] : 0.f);
+                Cf[e] = p.relu ? fmaxf(x, 0.f) : x;
+              }
+            }
+          } else if (VEC) {
+            typename Vec<T>::v4 o;
+            if (bias) {
+              const typename Vec<T>::v4 bv = *reinterpret_cast<const typename Vec<T>::v4*>(bias + n);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) v[e] += (float)bv[e];
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = (T)(p.relu ? fmaxf(v[e], 0.f) : v[e]);
+            *reinterpret_cast<typename Vec<T>::v4*>(C + (int64_t)m * p.ldc + n) = o;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              if (n + e < p.N) {
+                float x = v[e] + (bias ? (float)bias[n + e] : 0.f);
+                C[(int64_t)m * p.ldc + n + e] = (T)(p.relu ? fmaxf(x, 0.f) : x);
+              }
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
 template <typename T, int BM, int BN, int BK, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, bool VEC>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_kernel(GemmParams p) {
   constexpr int NT = WM * WN * 64;
@@ -137,7 +203,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_kernel(GemmParams p) {
 
   // ---- which tile / which slice of the contraction -------------------------
   const int tiles = p.tiles_m * p.tiles_n;
-  const int pid = remap_xcd(blockIdx.x, tiles * p.splits);
+  const int pid = (p.flags & 1) ? (int)blockIdx.x : remap_xcd(blockIdx.x, tiles * p.splits);
   const int split = pid / tiles;
   const int t = pid - split * tiles;
   const int per_group = GROUP_M * p.tiles_n;
@@ -202,70 +268,295 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_kernel(GemmParams p) {
     __syncthreads();
   }
 
-  // ---- epilogue: lane holds C[m][n .. n+3] for m = .. + lane%32 ------------
+  gemm_epilogue<T, TM, TN, WTM, WTN, VEC>(p, acc, m0, n0, wm, wn, lane, split);
+}
+
+
+// ---------------------------------------------------------------------------
+// Fast path: HBM -> LDS directly (global_load_lds_dwordx4, no VGPR round trip),
+// STAGES LDS buffers, loads issued STAGES-1 steps ahead of their use.
+// A wave-level load writes 64 x 16 bytes to consecutive LDS addresses, so the
+// chunk swizzle is applied on the GLOBAL side: the lane that owns LDS slot
+// (row, c') fetches chunk c = c' ^ swz(row).  Rows / columns beyond M / N are
+// clamped to valid memory (their products only reach C entries that are never
+// stored); the contraction extent must be a multiple of BK.
+// ---------------------------------------------------------------------------
+typedef __attribute__((address_space(1))) const void gptr_void;
+
+template <typename T, int R, int BK, bool KMAJOR, int NW>
+struct DmaPanel {
+  static constexpr int CPR = KMAJOR ? BK / 8 : R / 8;
+  static constexpr int LROWS = KMAJOR ? R : BK;
+  static constexpr int NCHUNK = LROWS * CPR;
+  static constexpr int BYTES = NCHUNK * 16;
+  static constexpr int WLOADS = NCHUNK / 64;   // wave-level loads per panel
+  static constexpr int PER_WAVE = WLOADS / NW;
+  static_assert(WLOADS % NW == 0 && PER_WAVE >= 1, "panel must divide evenly over the waves");
+  static_assert(KMAJOR ? (CPR == 4 || CPR == 8) : (CPR >= 16), "unsupported panel shape");
+
+  static __device__ __forceinline__ int swz(int lrow, int c) {
+    if (KMAJOR) return c ^ ((lrow / (16 / CPR)) % CPR);
+    return c ^ ((lrow & 3) << 2);
+  }
+
+  // Global address of each of this lane's chunks for the step starting at kbeg.
+  static __device__ __forceinline__ void init(const T* (&ptrs)[PER_WAVE], const T* base, int64_t ld, int row0,
+                                              int rmax, int kbeg, int wave, int lane) {
+#pragma unroll
+    for (int j = 0; j < PER_WAVE; ++j) {
+      const int slot = (wave * PER_WAVE + j) * 64 + lane;
+      const int lrow = slot / CPR;
+      const int c = swz(lrow, slot % CPR);
+      if (KMAJOR) {
+        const int gr = min(row0 + lrow, rmax - 1);
+        ptrs[j] = base + (int64_t)gr * ld + kbeg + c * 8;
+      } else {
+        int gr = row0 + c * 8;
+        if (gr >= rmax) gr = row0;
+        ptrs[j] = base + (int64_t)(kbeg + lrow) * ld + gr;
+      }
+    }
+  }
+  static __device__ __forceinline__ void issue(const T* (&ptrs)[PER_WAVE], char* lds, int wave) {
+#pragma unroll
+    for (int j = 0; j < PER_WAVE; ++j)
+      __builtin_amdgcn_global_load_lds((gptr_void*)ptrs[j], (lds_void*)(lds + (wave * PER_WAVE + j) * 1024), 16, 0, 0);
+  }
+  static __device__ __forceinline__ void advance(const T* (&ptrs)[PER_WAVE], int64_t ld) {
+#pragma unroll
+    for (int j = 0; j < PER_WAVE; ++j) ptrs[j] += KMAJOR ? (int64_t)BK : (int64_t)BK * ld;
+  }
+  static __device__ __forceinline__ typename Vec<T>::v8 frag(const char* lds, int rb, int ks, int lane) {
+    return Panel<T, R, BK, KMAJOR, 64, true>::frag(lds, rb, ks, lane);
+  }
+};
+
+// s_waitcnt vmcnt(n) with the other counters unconstrained (gfx9 encoding).
+template <int N> __device__ __forceinline__ void wait_vmcnt() {
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+
+// Epilogue of the direct-to-LDS kernel.  Each wave rounds its accumulators (after
+// bias / ReLU), parks one 32-row block at a time in a private LDS region and
+// reads it back row-contiguously, so every global store instruction writes whole
+// 16-byte chunks of complete row segments (8 rows x 128 B for a 64-wide wave
+// tile) instead of 32 scattered 16-byte pieces.
+template <typename T, typename TO, int TM, int TN, int WTM, int WTN>
+__device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x16 (&acc)[TM][TN], char* smem, int m0,
+                                                  int n0, int wm, int wn, int wave, int lane) {
+  constexpr int ES = (int)sizeof(TO);
+  constexpr int ROWB = WTN * ES + 16;     // padded row pitch in bytes
+  constexpr int CH = WTN * ES / 16;       // 16-byte chunks per row
+  constexpr int RPI = 64 / CH;            // rows covered by one wave-wide access
+  constexpr int EPC = 16 / ES;            // elements per chunk
+  char* mine = smem + wave * (32 * ROWB);
   const T* bias = (const T*)p.bias;
-  T* C = (T*)p.C;
+  TO* C = (TO*)p.C;
+  const int nbase = n0 + wn * WTN;
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
-    const int m = m0 + wm * WTM + i * 32 + (lane & 31);
-    if (m >= p.M) continue;
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const int n = n0 + wn * WTN + j * 32 + g * 8 + (lane >> 5) * 4;
-        if (n >= p.N) continue;
+        const int nl = j * 32 + g * 8 + (lane >> 5) * 4;
         float v[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[e] = acc[i][j][g * 4 + e];
-        if (p.splits > 1) {
-          float* dst = p.partial + ((int64_t)split * p.M + m) * p.N + n;
-          if (VEC) {
-            f32x4 o = {v[0], v[1], v[2], v[3]};
-            *reinterpret_cast<f32x4*>(dst) = o;
-          } else {
+        if (bias && nbase + nl < p.N) {
+          const typename Vec<T>::v4 bv = *reinterpret_cast<const typename Vec<T>::v4*>(bias + nbase + nl);
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-              if (n + e < p.N) dst[e] = v[e];
-          }
+          for (int e = 0; e < 4; ++e) v[e] += (float)bv[e];
+        }
+        if (p.relu) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = fmaxf(v[e], 0.f);
+        }
+        if (ES == 4) {
+          f32x4 o = {v[0], v[1], v[2], v[3]};
+          *reinterpret_cast<f32x4*>(mine + (lane & 31) * ROWB + nl * 4) = o;
         } else {
-          if (VEC) {
-            typename Vec<T>::v4 o;
-            if (bias) {
-              const typename Vec<T>::v4 bv = *reinterpret_cast<const typename Vec<T>::v4*>(bias + n);
+          typename Vec<T>::v4 o;
 #pragma unroll
-              for (int e = 0; e < 4; ++e) v[e] += (float)bv[e];
-            }
-#pragma unroll
-            for (int e = 0; e < 4; ++e) o[e] = (T)(p.relu ? fmaxf(v[e], 0.f) : v[e]);
-            *reinterpret_cast<typename Vec<T>::v4*>(C + (int64_t)m * p.ldc + n) = o;
-          } else {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              if (n + e < p.N) {
-                float x = v[e] + (bias ? (float)bias[n + e] : 0.f);
-                C[(int64_t)m * p.ldc + n + e] = (T)(p.relu ? fmaxf(x, 0.f) : x);
-              }
-            }
-          }
+          for (int e = 0; e < 4; ++e) o[e] = (T)v[e];
+          *reinterpret_cast<typename Vec<T>::v4*>(mine + (lane & 31) * ROWB + nl * 2) = o;
         }
       }
+    }
+#pragma unroll
+    for (int rr = 0; rr < 32 / RPI; ++rr) {
+      const int r = rr * RPI + lane / CH, c = lane % CH;
+      const u32x4 val = lds_ld16(mine, r * ROWB + c * 16);
+      const int m = m0 + wm * WTM + i * 32 + r, n = nbase + c * EPC;
+      if (m < p.M && n < p.N) st16(C + (int64_t)m * p.ldc + n, val);
     }
   }
 }
 
+template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES, int WPE, bool A_KMAJOR, bool B_KMAJOR>
+__global__ __launch_bounds__(WM* WN * 64, WPE) void gemm_dma_kernel(GemmParams p) {
+  constexpr int NW = WM * WN;
+  constexpr int WTM = BM / WM, WTN = BN / WN;
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  constexpr int GROUP_M = 8;
+  constexpr int D = STAGES - 1;  // prefetch distance
+  typedef DmaPanel<T, BM, BK, A_KMAJOR, NW> PA;
+  typedef DmaPanel<T, BN, BK, B_KMAJOR, NW> PB;
+  typedef typename Vec<T>::v8 v8;
+  constexpr int STAGE = PA::BYTES + PB::BYTES;
+  constexpr int LPS = PA::PER_WAVE + PB::PER_WAVE;  // loads per wave per stage
+  static_assert(LPS * D < 64, "vmcnt range");
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+
+  const int tiles = p.tiles_m * p.tiles_n;
+  const int pid = (p.flags & 1) ? (int)blockIdx.x : remap_xcd(blockIdx.x, tiles * p.splits);
+  const int split = pid / tiles;
+  const int t = pid - split * tiles;
+  const int per_group = GROUP_M * p.tiles_n;
+  const int group = t / per_group;
+  const int first_m = group * GROUP_M;
+  const int gsz = min(p.tiles_m - first_m, GROUP_M);
+  const int tm = first_m + (t % per_group) % gsz;
+  const int tn = (t % per_group) / gsz;
+  const int m0 = tm * BM, n0 = tn * BN;
+  const int kbeg = split * p.k_per_split;
+  const int kend = min(p.K, kbeg + p.k_per_split);
+  const int nk = (kend - kbeg) / BK;
+
+  const T* pa[PA::PER_WAVE];
+  const T* pb[PB::PER_WAVE];
+  PA::init(pa, (const T*)p.A, p.lda, m0, p.M, kbeg, wave, lane);
+  PB::init(pb, (const T*)p.B, p.ldb, n0, p.N, kbeg, wave, lane);
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  // prologue: D steps in flight
+#pragma unroll
+  for (int s = 0; s < D; ++s) {
+    if (s < nk) {
+      PA::issue(pa, smem + s * STAGE, wave);
+      PB::issue(pb, smem + s * STAGE + PA::BYTES, wave);
+      PA::advance(pa, p.lda);
+      PB::advance(pb, p.ldb);
+    }
+  }
+
+  int stage = 0;        // stage holding step kt
+  int fill = D % STAGES;  // stage that step kt + D goes to
+  for (int kt = 0; kt < nk; ++kt) {
+    // this wave's loads of step kt have landed once at most the later steps' loads are outstanding
+    const int later = min(D - 1, nk - 1 - kt);
+    if (later >= 2) wait_vmcnt<LPS * 2>();
+    else if (later == 1) wait_vmcnt<LPS * (D >= 2 ? 1 : 0)>();
+    else wait_vmcnt<0>();
+    // Bare s_barrier: __syncthreads() would add a fence that drains every outstanding
+    // direct-to-LDS load.  The waits that matter are explicit: this wave's loads of
+    // step kt (above) and its LDS reads of step kt-1 (consumed by the MFMAs already).
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (kt + D < nk && !(p.flags & 2)) {
+      PA::issue(pa, smem + fill * STAGE, wave);
+      PB::issue(pb, smem + fill * STAGE + PA::BYTES, wave);
+      PA::advance(pa, p.lda);
+      PB::advance(pb, p.ldb);
+    }
+    const char* sa = smem + stage * STAGE;
+    const char* sb = sa + PA::BYTES;
+    if (p.flags & 4) continue;
+    // operands of contraction step ks+1 are read from LDS while the MFMAs of step ks run
+    v8 fa[2][TM], fb[2][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) fa[0][i] = PA::frag(sa, wm * WTM + i * 32, 0, lane);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) fb[0][j] = PB::frag(sb, wn * WTN + j * 32, 0, lane);
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      if (ks + 1 < BK / 16) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa[(ks + 1) & 1][i] = PA::frag(sa, wm * WTM + i * 32, ks + 1, lane);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fb[(ks + 1) & 1][j] = PB::frag(sb, wn * WTN + j * 32, ks + 1, lane);
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = mfma32(fb[ks & 1][j], fa[ks & 1][i], acc[i][j]);
+      // issue order within the step: the LDS reads of step ks+1 are spread between
+      // the MFMAs of step ks instead of being bunched in front of them
+      if (ks + 1 < BK / 16) {
+        constexpr int NREAD = TM * (A_KMAJOR ? 1 : 2) + TN * (B_KMAJOR ? 1 : 2);
+        constexpr int NMFMA = TM * TN;
+        constexpr int PER = NREAD >= NMFMA ? (NREAD + NMFMA - 1) / NMFMA : 1;  // reads after each MFMA
+        constexpr int SLOTS = (NREAD + PER - 1) / PER;
+#pragma unroll
+        for (int q = 0; q < SLOTS; ++q) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, PER, 0);
+        }
+        if (NMFMA > SLOTS) __builtin_amdgcn_sched_group_barrier(0x008, NMFMA - SLOTS, 0);
+      }
+    }
+    stage = stage + 1 == STAGES ? 0 : stage + 1;
+    fill = fill + 1 == STAGES ? 0 : fill + 1;
+  }
+
+  if (p.flags & 8) return;
+  if (p.splits > 1) {
+    gemm_epilogue<T, TM, TN, WTM, WTN, true>(p, acc, m0, n0, wm, wn, lane, split);
+  } else {
+    static_assert(NW * 32 * (WTN * 4 + 16) <= STAGES * STAGE, "epilogue staging must fit in the pipeline LDS");
+    __syncthreads();  // all waves are done reading the last pipeline stage
+    if (p.out_f32) gemm_epilogue_lds<T, float, TM, TN, WTM, WTN>(p, acc, smem, m0, n0, wm, wn, wave, lane);
+    else gemm_epilogue_lds<T, T, TM, TN, WTM, WTN>(p, acc, smem, m0, n0, wm, wn, wave, lane);
+  }
+}
+
 // Sum the split-contraction partials in a fixed order and apply the epilogue.
-template <typename T>
+// VEC4: N and ldc multiples of 4, 16-byte aligned partials, 8-byte aligned C.
+template <typename T, typename TO, bool VEC4>
 __global__ __launch_bounds__(256) void gemm_reduce(int M, int N, int splits, const float* __restrict__ partial,
-                                                    const T* __restrict__ bias, int relu, T* __restrict__ C,
+                                                    const T* __restrict__ bias, int relu, TO* __restrict__ C,
                                                     int64_t ldc) {
   const int64_t total = (int64_t)M * N;
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
-    float s = 0.f;
-    for (int k = 0; k < splits; ++k) s += partial[(int64_t)k * total + i];
-    const int m = (int)(i / N), n = (int)(i - (int64_t)m * N);
-    if (bias) s += (float)bias[n];
-    C[(int64_t)m * ldc + n] = (T)(relu ? fmaxf(s, 0.f) : s);
+  if (VEC4) {
+    const int64_t quads = total >> 2;
+    for (int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x; q < quads; q += (int64_t)gridDim.x * 256) {
+      f32x4 s = *reinterpret_cast<const f32x4*>(partial + q * 4);
+      for (int k = 1; k < splits; ++k) s += *reinterpret_cast<const f32x4*>(partial + (int64_t)k * total + q * 4);
+      const int64_t i = q * 4;
+      const int m = (int)(i / N), n = (int)(i - (int64_t)m * N);
+      TO o[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float x = s[e] + (bias ? (float)bias[n + e] : 0.f);
+        o[e] = (TO)(relu ? fmaxf(x, 0.f) : x);
+      }
+      struct alignas(sizeof(TO) * 4) Quad { TO v[4]; };
+      Quad qd;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) qd.v[e] = o[e];
+      *reinterpret_cast<Quad*>(C + (int64_t)m * ldc + n) = qd;
+    }
+  } else {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+      float s = 0.f;
+      for (int k = 0; k < splits; ++k) s += partial[(int64_t)k * total + i];
+      const int m = (int)(i / N), n = (int)(i - (int64_t)m * N);
+      if (bias) s += (float)bias[n];
+      C[(int64_t)m * ldc + n] = (TO)(relu ? fmaxf(s, 0.f) : s);
+    }
   }
 }
 
@@ -273,40 +564,69 @@ __global__ __launch_bounds__(256) void gemm_reduce(int M, int N, int splits, con
 // host side: tile choice, contraction split, launch
 // ---------------------------------------------------------------------------
 struct GemmPlan {
-  int cfg;  // 0: 256x256x64 / 8 waves, 1: 128x128x64 / 4 waves
+  int cfg;
   int bm, bn, bk;
   int tiles_m, tiles_n, splits, k_per_split;
 };
+
+struct TileCfg { int bm, bn, bk, waves, stages; };  // stages > 0: direct-to-LDS kernel
+// index = cfg id used by launch_cfg below
+static const TileCfg kCfgs[] = {
+    {256, 256, 64, 8, 0},  // 0: register-staged, wave tile 128x64
+    {128, 128, 64, 4, 0},  // 1: register-staged, wave tile 64x64
+    {256, 256, 32, 8, 4},  // 2: direct-to-LDS, 4 stages, wave tile 128x64
+    {256, 128, 32, 4, 4},  // 3: direct-to-LDS, 4 stages, wave tile 128x64
+    {256, 256, 32, 8, 3},  // 4
+    {128, 128, 32, 4, 4},  // 5: wave tile 64x64
+    {256, 128, 64, 4, 3},  // 6
+    {256, 256, 64, 8, 2},  // 7
+    {128, 128, 64, 4, 2},  // 8: 64 KB LDS, two workgroups per CU
+    {256, 128, 32, 4, 3},  // 9: 72 KB LDS, two workgroups per CU, wave tile 128x64
+    {128, 256, 32, 4, 3},  // 10: as 9, wave tile 64x128
+    {128, 128, 64, 4, 3},  // 11
+};
+constexpr int kNumCfgs = (int)(sizeof(kCfgs) / sizeof(kCfgs[0]));
 
 static int env_int(const char* name, int dflt) {
   const char* s = getenv(name);
   return s ? atoi(s) : dflt;
 }
+static int g_force_cfg = env_int("TF_GEMM_CFG", -1);
+static int g_force_splits = env_int("TF_GEMM_SPLITS", 0);
+static int g_flags = env_int("TF_GEMM_FLAGS", 0);
 
-static GemmPlan make_plan(int64_t M, int64_t N, int64_t K) {
-  static const int force_cfg = env_int("TF_GEMM_CFG", -1);
-  static const int force_splits = env_int("TF_GEMM_SPLITS", 0);
+static GemmPlan make_plan(int64_t M, int64_t N, int64_t K, bool vec) {
   GemmPlan pl;
   const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
-  pl.cfg = big_tiles >= 192 ? 0 : 1;
-  if (force_cfg >= 0 && force_cfg <= 1) pl.cfg = force_cfg;
-  pl.bm = pl.bn = pl.cfg == 0 ? 256 : 128;
-  pl.bk = 64;
+  // Measured on MI355X (gfx950): 256x256 tiles win once they alone give every CU
+  // work, and for long contractions over a mid-sized output (weight gradients of
+  // the MLP) when combined with a contraction split; everything else runs
+  // 128x128 tiles with two workgroups resident per CU.
+  const bool dma = vec && K % 64 == 0;
+  const bool long_k_mid = big_tiles >= 48 && big_tiles < 128 && K >= 4096 && K >= 2 * (M > N ? M : N);
+  if (big_tiles >= 200 || long_k_mid) pl.cfg = dma ? 7 : 0;
+  else pl.cfg = dma ? 8 : 1;
+  if (g_force_cfg >= 0 && g_force_cfg < kNumCfgs) pl.cfg = g_force_cfg;
+  if (kCfgs[pl.cfg].stages > 0 && !(vec && K % kCfgs[pl.cfg].bk == 0))
+    pl.cfg = kCfgs[pl.cfg].bm * kCfgs[pl.cfg].bn >= 256 * 256 ? 0 : 1;  // register-staged twin
+  pl.bm = kCfgs[pl.cfg].bm;
+  pl.bn = kCfgs[pl.cfg].bn;
+  pl.bk = kCfgs[pl.cfg].bk;
   pl.tiles_m = (int)((M + pl.bm - 1) / pl.bm);
   pl.tiles_n = (int)((N + pl.bn - 1) / pl.bn);
   const int64_t tiles = (int64_t)pl.tiles_m * pl.tiles_n;
   const int64_t ksteps = (K + pl.bk - 1) / pl.bk;
-  // Split the contraction only when the tile count alone cannot fill 256 CUs
-  // and each slice still keeps at least 8 steps of work.
+  // Split the contraction only when the tiles alone leave most CUs idle (weight
+  // gradients of square layers: few output tiles, long contraction); every slice
+  // keeps at least 16 steps so the fp32 partial traffic stays small.
   int64_t splits = 1;
-  const int64_t target = pl.cfg == 0 ? 256 : 512;
-  if (tiles < target) {
-    splits = (target + tiles - 1) / tiles;
-    const int64_t max_by_k = ksteps / 8 > 0 ? ksteps / 8 : 1;
+  if (tiles < 128) {
+    splits = (256 + tiles - 1) / tiles;
+    const int64_t max_by_k = ksteps / 16 > 0 ? ksteps / 16 : 1;
     if (splits > max_by_k) splits = max_by_k;
-    if (splits > 32) splits = 32;
+    if (splits > 16) splits = 16;
   }
-  if (force_splits > 0) splits = force_splits;
+  if (g_force_splits > 0) splits = g_force_splits;
   if (splits > ksteps) splits = ksteps > 0 ? ksteps : 1;
   const int64_t steps_per = (ksteps + splits - 1) / splits;
   pl.k_per_split = (int)(steps_per * pl.bk);
@@ -335,10 +655,43 @@ static int launch_one(hipStream_t st, const GemmParams& p) {
   return TF_OK;
 }
 
+template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES, int WPE, bool AK, bool BKM>
+static int launch_dma(hipStream_t st, const GemmParams& p) {
+  constexpr int lds = STAGES * (BM + BN) * BK * 2;
+  static_assert(lds <= 160 * 1024, "LDS budget");
+  auto kernel = gemm_dma_kernel<T, BM, BN, BK, WM, WN, STAGES, WPE, AK, BKM>;
+  static bool once = (allow_big_lds(kernel, lds), true);
+  (void)once;
+  const unsigned grid = (unsigned)(p.tiles_m * p.tiles_n * p.splits);
+  kernel<<<dim3(grid), dim3(WM * WN * 64), lds, st>>>(p);
+  TF_CHECK_LAUNCH();
+  return TF_OK;
+}
+
+// The register-staged kernel handles everything (ragged extents, unaligned
+// pointers); the direct-to-LDS kernel needs the vector conditions and a
+// contraction extent that is a multiple of its BK.
 template <typename T, bool AK, bool BKM, bool VEC>
 static int launch_cfg(hipStream_t st, const GemmPlan& pl, const GemmParams& p) {
-  if (pl.cfg == 0) return launch_one<T, 256, 256, 64, 2, 4, AK, BKM, VEC>(st, p);
-  return launch_one<T, 128, 128, 64, 2, 2, AK, BKM, VEC>(st, p);
+  const bool dma_ok = VEC && p.K % pl.bk == 0;
+  if (kCfgs[pl.cfg].stages > 0 && dma_ok) {
+    switch (pl.cfg) {
+      case 2: return launch_dma<T, 256, 256, 32, 2, 4, 4, 2, AK, BKM>(st, p);
+      case 3: return launch_dma<T, 256, 128, 32, 2, 2, 4, 1, AK, BKM>(st, p);
+      case 4: return launch_dma<T, 256, 256, 32, 2, 4, 3, 2, AK, BKM>(st, p);
+      case 5: return launch_dma<T, 128, 128, 32, 2, 2, 4, 2, AK, BKM>(st, p);
+      case 6: return launch_dma<T, 256, 128, 64, 2, 2, 3, 1, AK, BKM>(st, p);
+      case 7: return launch_dma<T, 256, 256, 64, 2, 4, 2, 2, AK, BKM>(st, p);
+      case 8: return launch_dma<T, 128, 128, 64, 2, 2, 2, 2, AK, BKM>(st, p);
+      case 9: return launch_dma<T, 256, 128, 32, 2, 2, 3, 2, AK, BKM>(st, p);
+      case 10: return launch_dma<T, 128, 256, 32, 2, 2, 3, 2, AK, BKM>(st, p);
+      case 11: return launch_dma<T, 128, 128, 64, 2, 2, 3, 1, AK, BKM>(st, p);
+    }
+  }
+  // fallbacks with the same tile shape where one exists
+  if (pl.bm == 256 && pl.bn == 256 && pl.bk == 64) return launch_one<T, 256, 256, 64, 2, 4, AK, BKM, VEC>(st, p);
+  if (pl.bm == 128 && pl.bn == 128 && pl.bk == 64) return launch_one<T, 128, 128, 64, 2, 2, AK, BKM, VEC>(st, p);
+  return TF_EINVAL;
 }
 
 template <typename T>
@@ -354,10 +707,17 @@ static int gemm_dispatch(hipStream_t st, int la, int lb, bool vec, const GemmPla
   if (rc != TF_OK) return rc;
   if (p.splits > 1) {
     const int64_t total = (int64_t)p.M * p.N;
-    int64_t blocks = (total + 255) / 256;
-    if (blocks > 8192) blocks = 8192;
-    gemm_reduce<T><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(p.M, p.N, p.splits, p.partial, (const T*)p.bias,
-                                                                 p.relu, (T*)p.C, p.ldc);
+    const bool v4 = p.N % 4 == 0 && p.ldc % 4 == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0;
+    int64_t blocks = ((v4 ? total / 4 : total) + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    if (blocks < 1) blocks = 1;
+    const dim3 g((unsigned)blocks), b(256);
+    const T* bias = (const T*)p.bias;
+#define REDUCE(TO, V4) \
+  gemm_reduce<T, TO, V4><<<g, b, 0, st>>>(p.M, p.N, p.splits, p.partial, bias, p.relu, (TO*)p.C, p.ldc)
+    if (p.out_f32) { if (v4) REDUCE(float, true); else REDUCE(float, false); }
+    else { if (v4) REDUCE(T, true); else REDUCE(T, false); }
+#undef REDUCE
     TF_CHECK_LAUNCH();
   }
   return TF_OK;
@@ -367,18 +727,47 @@ static int gemm_dispatch(hipStream_t st, int la, int lb, bool vec, const GemmPla
 
 using namespace tfa;
 
+// Diagnostic: force a tile configuration (index into kCfgs, -1 = automatic) and
+// a contraction split (0 = automatic) for every later tf_gemm call.
+extern "C" int tf_gemm_tune(int cfg, int splits) {
+  if (cfg >= kNumCfgs) return TF_EINVAL;
+  g_force_cfg = cfg;
+  g_force_splits = splits;
+  return TF_OK;
+}
+
+// Diagnostic: bit 0 skips the XCD remap, bit 1 skips the in-loop loads, bit 2 the MFMA work.
+extern "C" int tf_gemm_debug_flags(int flags) {
+  g_flags = flags;
+  return TF_OK;
+}
+
 extern "C" int64_t tf_gemm_workspace_bytes(int layout_a, int layout_b, int64_t M, int64_t N, int64_t K) {
   (void)layout_a;
   (void)layout_b;
   if (M <= 0 || N <= 0 || K <= 0) return 0;
-  const GemmPlan pl = make_plan(M, N, K);
-  return pl.splits > 1 ? (int64_t)pl.splits * M * N * (int64_t)sizeof(float) : 0;
+  // the caller's alignment is unknown here: cover both kernel families
+  int64_t need = 0;
+  for (int vec = 0; vec < 2; ++vec) {
+    const GemmPlan pl = make_plan(M, N, K, vec != 0);
+    const int64_t n = pl.splits > 1 ? (int64_t)pl.splits * M * N * (int64_t)sizeof(float) : 0;
+    if (n > need) need = n;
+  }
+  return need;
 }
 
 extern "C" int tf_gemm(void* stream, int dtype, int layout_a, int layout_b, int64_t M, int64_t N, int64_t K,
                        const void* A, int64_t lda, const void* B, int64_t ldb, void* C, int64_t ldc,
                        const void* bias, int relu, void* workspace, int64_t workspace_bytes) {
+  return tf_gemm_out(stream, dtype, dtype, layout_a, layout_b, M, N, K, A, lda, B, ldb, C, ldc, bias, relu, workspace,
+                     workspace_bytes);
+}
+
+extern "C" int tf_gemm_out(void* stream, int dtype, int out_dtype, int layout_a, int layout_b, int64_t M, int64_t N,
+                           int64_t K, const void* A, int64_t lda, const void* B, int64_t ldb, void* C, int64_t ldc,
+                           const void* bias, int relu, void* workspace, int64_t workspace_bytes) {
   if (!A || !B || !C) return TF_EINVAL;
+  if (out_dtype != dtype && out_dtype != TF_F32) return TF_EDTYPE;
   if (M <= 0 || N <= 0 || K <= 0 || M > 0x7fffff00 || N > 0x7fffff00 || K > 0x7fffff00) return TF_EINVAL;
   if ((layout_a != TF_OP_KMAJOR && layout_a != TF_OP_KMINOR) || (layout_b != TF_OP_KMAJOR && layout_b != TF_OP_KMINOR))
     return TF_EINVAL;
@@ -390,14 +779,13 @@ extern "C" int tf_gemm(void* stream, int dtype, int layout_a, int layout_b, int6
        reinterpret_cast<uintptr_t>(bias)) & 1)
     return TF_EALIGN;
 
-  const GemmPlan pl = make_plan(M, N, K);
+  const bool vec = aligned16(A) && aligned16(B) && aligned16(C) && (!bias || aligned16(bias)) && a_contig % 8 == 0 &&
+                   b_contig % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 && N % 8 == 0 && ldc % 8 == 0;
+  const GemmPlan pl = make_plan(M, N, K, vec);
   const int64_t need = pl.splits > 1 ? (int64_t)pl.splits * M * N * (int64_t)sizeof(float) : 0;
   if (need > 0 && (!workspace || workspace_bytes < need)) return TF_EWORKSPACE;
   if (need > 0 && !aligned16(workspace)) return TF_EALIGN;
   if ((int64_t)pl.tiles_m * pl.tiles_n * pl.splits > 0x7fffffff) return TF_EINVAL;
-
-  const bool vec = aligned16(A) && aligned16(B) && aligned16(C) && (!bias || aligned16(bias)) && a_contig % 8 == 0 &&
-                   b_contig % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 && N % 8 == 0 && ldc % 8 == 0;
 
   GemmParams p;
   p.A = A; p.B = B; p.C = C; p.bias = bias; p.partial = (float*)workspace;
@@ -406,6 +794,8 @@ extern "C" int tf_gemm(void* stream, int dtype, int layout_a, int layout_b, int6
   p.relu = relu ? 1 : 0;
   p.splits = pl.splits; p.k_per_split = pl.k_per_split;
   p.tiles_m = pl.tiles_m; p.tiles_n = pl.tiles_n;
+  p.flags = g_flags;
+  p.out_f32 = out_dtype == TF_F32 ? 1 : 0;
   hipStream_t st = (hipStream_t)stream;
   if (dtype == TF_F16) return gemm_dispatch<f16>(st, layout_a, layout_b, vec, pl, p);
   return gemm_dispatch<bf16>(st, layout_a, layout_b, vec, pl, p);

@@ -211,28 +211,26 @@ __global__ __launch_bounds__(256) void ln_bwd_any(int64_t rows, int d, const T* 
   }
 }
 
-// Second stage: dgamma[c] = sum_b partial[b][0][c], dbeta[c] = sum_b partial[b][1][c].
-// Workgroup = 64 columns x 4 slices of the partial rows.
+// Second stage over partial viewed as a [nparts][2d] matrix (dgamma columns then
+// dbeta columns): workgroup = 16 columns x 16 row slices, slices summed in a
+// fixed order through LDS.
 template <typename T>
 __global__ __launch_bounds__(256) void ln_bwd_reduce(int nparts, int d, const float* __restrict__ partial,
                                                       T* __restrict__ dgamma, T* __restrict__ dbeta) {
-  __shared__ float red[2][4][64];
-  const int col = blockIdx.x * 64 + (threadIdx.x & 63);
-  const int slice = threadIdx.x >> 6;
-  float a = 0.f, b = 0.f;
-  if (col < d) {
-    for (int p = slice; p < nparts; p += 4) {
-      a += partial[(int64_t)p * 2 * d + col];
-      b += partial[(int64_t)p * 2 * d + d + col];
-    }
-  }
-  red[0][slice][threadIdx.x & 63] = a;
-  red[1][slice][threadIdx.x & 63] = b;
+  __shared__ float red[16][17];
+  const int cl = threadIdx.x & 15, slice = threadIdx.x >> 4;
+  const int col = blockIdx.x * 16 + cl;  // 0 .. 2d-1
+  float a = 0.f;
+  if (col < 2 * d)
+    for (int p = slice; p < nparts; p += 16) a += partial[(int64_t)p * 2 * d + col];
+  red[slice][cl] = a;
   __syncthreads();
-  if (slice == 0 && col < d) {
-    const int l = threadIdx.x;
-    dgamma[col] = (T)(red[0][0][l] + red[0][1][l] + red[0][2][l] + red[0][3][l]);
-    dbeta[col] = (T)(red[1][0][l] + red[1][1][l] + red[1][2][l] + red[1][3][l]);
+  if (slice == 0 && col < 2 * d) {
+    float s = 0.f;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) s += red[k][cl];
+    if (col < d) dgamma[col] = (T)s;
+    else dbeta[col - d] = (T)s;
   }
 }
 
@@ -409,7 +407,7 @@ static int ln_bwd_launch(hipStream_t st, int64_t rows, int64_t d, const void* dy
   }
 #undef LN_BWD
   TF_CHECK_LAUNCH();
-  ln_bwd_reduce<T><<<dim3(ceil_div(d, 64)), dim3(256), 0, st>>>(parts, (int)d, partial, (T*)dgamma, (T*)dbeta);
+  ln_bwd_reduce<T><<<dim3(ceil_div(2 * d, 16)), dim3(256), 0, st>>>(parts, (int)d, partial, (T*)dgamma, (T*)dbeta);
   TF_CHECK_LAUNCH();
   return TF_OK;
 }

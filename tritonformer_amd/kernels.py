@@ -32,9 +32,9 @@ def _gemm(dtype, la, lb, m, n, k, a, lda, b, ldb, c, ldc, bias, relu):
     lib = load()
     ws_bytes = _gemm_ws(la, lb, m, n, k)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=c.device) if ws_bytes else None
-    check(lib.tf_gemm(stream_ptr(), dtype_code(dtype), la, lb, m, n, k, a.data_ptr(), lda, b.data_ptr(), ldb,
-                      c.data_ptr(), ldc, bias.data_ptr() if bias is not None else None, int(relu),
-                      ws.data_ptr() if ws is not None else None, ws_bytes))
+    check(lib.tf_gemm_out(stream_ptr(), dtype_code(dtype), dtype_code(c.dtype), la, lb, m, n, k, a.data_ptr(), lda,
+                          b.data_ptr(), ldb, c.data_ptr(), ldc, bias.data_ptr() if bias is not None else None,
+                          int(relu), ws.data_ptr() if ws is not None else None, ws_bytes))
 
 
 def _check_linear(a, b, bias=None):
@@ -74,10 +74,12 @@ def mm(a, b, fuse_relu=False):
     return gemm(a, b, None, fuse_relu)
 
 
-def mm_dw(x, grad):
+def mm_dw(x, grad, out_dtype=None):
     """``sum_b x[b]^T @ grad[b]`` -> (in, out): reference ``bmm`` of the
     transposed view (kernels/gemm.py:161-200) followed by ``torch.sum`` over the
-    batch (linear.py:24-25), as ONE contraction over all B*S tokens."""
+    batch (linear.py:24-25), as ONE contraction over all B*S tokens.
+    ``out_dtype=torch.float32`` stores the fp32 accumulators unrounded (gradient
+    of an fp32 master weight)."""
     if x.shape[:-1] != grad.shape[:-1]:
         raise ValueError("Leading dimensions of the two operands do not match")
     if x.dtype != grad.dtype:
@@ -85,7 +87,7 @@ def mm_dw(x, grad):
     require_cuda(x, grad)
     x2, t, kin = _rows2d(x)
     g2, _, nout = _rows2d(grad)
-    out = torch.empty((kin, nout), dtype=x.dtype, device=x.device)
+    out = torch.empty((kin, nout), dtype=out_dtype or x.dtype, device=x.device)
     _gemm(x.dtype, KMINOR, KMINOR, kin, nout, t, x2, kin, g2, nout, out, nout, None, False)
     return out
 

@@ -12,7 +12,12 @@ def _grads(ctx, grad_output, inputs, weights):
     dW = X^T dY with the batch folded into the contraction
     (reference linear.py:21-25 goes through bmm + torch.sum)."""
     grad_input = mm(grad_output, weights.T) if ctx.needs_input_grad[0] else None
-    grad_weights = mm_dw(inputs, grad_output) if ctx.needs_input_grad[1] else None
+    grad_weights = None
+    if ctx.needs_input_grad[1]:
+        # an fp32 master weight (cast to 16 bit by autocast on the way in) gets its
+        # gradient straight from the fp32 accumulators instead of a rounded copy
+        master = torch.float32 if ctx.arg_dtypes[1] == torch.float32 else None
+        grad_weights = mm_dw(inputs, grad_output, out_dtype=master)
     return grad_input, grad_weights
 
 

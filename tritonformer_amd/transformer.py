@@ -179,8 +179,12 @@ class Transformer(nn.Module):
             positions = torch.arange(seq_len, device=hidden_states.device)[None].expand(batch_size, -1)
             hidden_states = hidden_states + self.embed_positions(positions)
         attn_bias = self.attn_bias
-        if attn_bias is not None and torch.is_autocast_enabled("cuda"):
-            attn_bias = attn_bias.to(torch.get_autocast_dtype("cuda"))
+        if torch.is_autocast_enabled("cuda"):
+            # keep the residual stream in the 16-bit compute type, as it is in the
+            # reference (whose embeddings are fp16 parameters, transformer.py:259-272)
+            hidden_states = hidden_states.to(torch.get_autocast_dtype("cuda"))
+            if attn_bias is not None:
+                attn_bias = attn_bias.to(torch.get_autocast_dtype("cuda"))
         for layer in self.layer_list:
             hidden_states = layer(hidden_states, attn_bias)
         hidden_states = self.final_layernorm(hidden_states)
