@@ -18,6 +18,7 @@
 //     ds_read_b64_tr_b16.
 // The 16 contraction slots of lane-half h in step t map to sequence offsets
 // 16t + 8(s/4) + 4h + s%4 (s = 0..7), on both operands alike.
+#include <type_traits>
 #include "rowops.h"
 
 namespace tfa {
@@ -105,9 +106,19 @@ __device__ __forceinline__ int reg_row(int r, int lane) { return (r >> 2) * 8 + 
 
 // ===========================================================================
 // Forward.  Workgroup: 4 waves x 32 queries; key/value blocks of 64.
+//
+// The softmax arithmetic runs on the VALU and is what bounds this kernel, so it
+// is kept to ~6 operations per score: one fma folds scale (and bias) into the
+// exp2 argument, the running maximum is only raised (and the accumulators
+// rescaled) when a row's maximum grew by more than 2^8 -- probabilities then
+// stay below 256, exact in 16 bit -- the causal mask is only evaluated on
+// blocks that touch the diagonal, and the row sums are produced by the matrix
+// core (an all-ones operand against P) instead of 32 VALU adds per row.
 // ===========================================================================
+constexpr float kRescaleThreshold = 8.0f;  // log2 domain
+
 template <typename T, int HD, bool HAS_BIAS>
-__global__ __launch_bounds__(256) void attn_fwd_kernel(AttnParams p) {
+__global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_fwd_kernel(AttnParams p) {
   typedef SeqTile<T, 64, HD> KT;
   typedef typename Vec<T>::v8 v8;
   typedef typename Vec<T>::v4 v4;
@@ -133,6 +144,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnParams p) {
   const int myq = q0w + (lane & 31);
   const int kv_end = min(p.S, q0 + 128);
   const int nkv = kv_end / 64;
+  const T* bias_row = HAS_BIAS ? (const T*)p.bias + (int64_t)h * p.bias_sh + (int64_t)myq * p.bias_sr : nullptr;
 
   v8 qf[KS];
 #pragma unroll
@@ -141,13 +153,18 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnParams p) {
     if (active) raw = ld16(Q + (int64_t)myq * p.ss + ks * 16 + (lane >> 5) * 8);
     qf[ks] = __builtin_bit_cast(v8, raw);
   }
+  v8 ones;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) ones[e] = (T)1.0f;
 
-  f32x16 oacc[DT];
+  f32x16 oacc[DT], lacc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) lacc[r] = 0.f;
 #pragma unroll
   for (int d = 0; d < DT; ++d)
 #pragma unroll
     for (int r = 0; r < 16; ++r) oacc[d][r] = 0.f;
-  float m_run = -INFINITY, l_run = 0.f;
+  float m_ref = -INFINITY;  // reference maximum (log2 domain) the accumulators are scaled to
 
   u32x4 rk[KT::PER_THREAD], rv[KT::PER_THREAD];
   KT::fetch(rk, K, p.ss, 0);
@@ -166,72 +183,76 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnParams p) {
     }
     const int kb = j * 64;
     if (active && kb <= q0w + 31) {
-      const bool live1 = kb + 32 <= q0w + 31;  // second 32-key half not fully above the diagonal
-      f32x16 st[2];
+      auto block = [&](auto diag_tag) {
+        constexpr bool DIAG = decltype(diag_tag)::value;
+        // on a diagonal block the second 32-key half may lie entirely above the diagonal
+        const bool live1 = !DIAG || kb + 32 <= q0w + 31;
+        f32x16 st[2];
 #pragma unroll
-      for (int jt = 0; jt < 2; ++jt) {
+        for (int jt = 0; jt < 2; ++jt) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) st[jt][r] = 0.f;
-        if (jt == 0 || live1) {
+          for (int r = 0; r < 16; ++r) st[jt][r] = 0.f;
+          if (jt == 0 || live1) {
 #pragma unroll
-          for (int ks = 0; ks < KS; ++ks) st[jt] = mfma32(KT::frag_rows(sk, jt * 32, ks, lane), qf[ks], st[jt]);
-        }
-      }
-      // scale, bias, causal mask; running max
-      float mx = -INFINITY;
-#pragma unroll
-      for (int jt = 0; jt < 2; ++jt) {
-        const bool live = jt == 0 || live1;
-        const bool diag = kb + jt * 32 + 31 > q0w;
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const int key0 = kb + jt * 32 + g * 8 + 4 * (lane >> 5);
-          float bv[4] = {0.f, 0.f, 0.f, 0.f};
-          if (HAS_BIAS && live) {
-            const v4 raw = *reinterpret_cast<const v4*>((const T*)p.bias + (int64_t)h * p.bias_sh +
-                                                        (int64_t)myq * p.bias_sr + key0);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) bv[e] = (float)raw[e] * kLog2e;
-          }
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            float s = st[jt][g * 4 + e] * p.scale_log2 + bv[e];
-            if (!live || (diag && key0 + e > myq)) s = -INFINITY;
-            st[jt][g * 4 + e] = s;
-            mx = fmaxf(mx, s);
+            for (int ks = 0; ks < KS; ++ks) st[jt] = mfma32(KT::frag_rows(sk, jt * 32, ks, lane), qf[ks], st[jt]);
           }
         }
-      }
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m_run, mx);
-      const float m_use = m_new == -INFINITY ? 0.f : m_new;
-      const float alpha = fast_exp2(m_run - m_use);
-      m_run = m_new;
-      float rs = 0.f;
+        // x = s * scale * log2e (+ bias * log2e), masked; block maximum
+        float mx = -INFINITY;
 #pragma unroll
-      for (int jt = 0; jt < 2; ++jt)
+        for (int jt = 0; jt < 2; ++jt) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float e = fast_exp2(st[jt][r] - m_use);
-          st[jt][r] = e;
-          rs += e;
-        }
-      l_run = l_run * alpha + rs;
+          for (int g = 0; g < 4; ++g) {
+            const int key0 = kb + jt * 32 + g * 8 + 4 * (lane >> 5);
+            float bv[4] = {0.f, 0.f, 0.f, 0.f};
+            if (HAS_BIAS && (jt == 0 || live1)) {
+              const v4 raw = *reinterpret_cast<const v4*>(bias_row + key0);
 #pragma unroll
-      for (int d = 0; d < DT; ++d)
+              for (int e = 0; e < 4; ++e) bv[e] = (float)raw[e] * kLog2e;
+            }
 #pragma unroll
-        for (int r = 0; r < 16; ++r) oacc[d][r] *= alpha;
-#pragma unroll
-      for (int jt = 0; jt < 2; ++jt) {
-        if (jt == 0 || live1) {
-#pragma unroll
-          for (int t = 0; t < 2; ++t) {
-            const v8 pb = round8<T>(st[jt], t);
-#pragma unroll
-            for (int d = 0; d < DT; ++d) oacc[d] = mfma32(KT::frag_hd(sv, jt * 32 + t * 16, d, lane), pb, oacc[d]);
+            for (int e = 0; e < 4; ++e) {
+              float x = HAS_BIAS ? fmaf(st[jt][g * 4 + e], p.scale_log2, bv[e]) : st[jt][g * 4 + e] * p.scale_log2;
+              if (DIAG && (key0 + e > myq || (jt == 1 && !live1))) x = -INFINITY;
+              st[jt][g * 4 + e] = x;
+              mx = fmaxf(mx, x);
+            }
           }
         }
-      }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        // raise the reference maximum only when some row outgrew it by 2^8
+        const bool grow = mx > m_ref + kRescaleThreshold;
+        if (__any(grow)) {
+          const float m_new = grow ? mx : m_ref;
+          const float alpha = grow ? fast_exp2(m_ref - m_new) : 1.0f;  // exp2(-inf) = 0 on the first block
+          m_ref = m_new;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) lacc[r] *= alpha;
+#pragma unroll
+          for (int d = 0; d < DT; ++d)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[d][r] *= alpha;
+        }
+        const float m_use = m_ref == -INFINITY ? 0.f : m_ref;  // row with nothing but -inf so far
+#pragma unroll
+        for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) st[jt][r] = fast_exp2(st[jt][r] - m_use);
+#pragma unroll
+        for (int jt = 0; jt < 2; ++jt) {
+          if (jt == 0 || live1) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+              const v8 pb = round8<T>(st[jt], t);
+              lacc = mfma32(ones, pb, lacc);  // every row of lacc = sum over keys of P
+#pragma unroll
+              for (int d = 0; d < DT; ++d) oacc[d] = mfma32(KT::frag_hd(sv, jt * 32 + t * 16, d, lane), pb, oacc[d]);
+            }
+          }
+        }
+      };
+      if (kb + 63 > q0w) block(std::true_type{});
+      else block(std::false_type{});
     }
     if (more) {
       char* dk = smem + ((j + 1) & 1) * STAGE;
@@ -242,9 +263,9 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnParams p) {
   }
 
   if (active) {
-    const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+    const float l_tot = lacc[0];
     const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-    if (lane < 32) p.lse[(int64_t)bh * p.S + myq] = m_run + log2f(l_tot);
+    if (lane < 32) p.lse[(int64_t)bh * p.S + myq] = m_ref + log2f(l_tot);
 #pragma unroll
     for (int d = 0; d < DT; ++d)
 #pragma unroll
@@ -286,7 +307,7 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(AttnParams p) {
 // diagonal downwards.  Q and dO tiles (+ their lse / delta) go through LDS.
 // ===========================================================================
 template <typename T, int HD, bool HAS_BIAS>
-__global__ __launch_bounds__(256) void attn_dkdv_kernel(AttnParams p) {
+__global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_dkdv_kernel(AttnParams p) {
   typedef SeqTile<T, 64, HD> QT;
   typedef typename Vec<T>::v8 v8;
   typedef typename Vec<T>::v4 v4;
@@ -331,13 +352,13 @@ __global__ __launch_bounds__(256) void attn_dkdv_kernel(AttnParams p) {
 
   const int nq = (p.S - k0) / 64;  // query blocks k0, k0+64, ...
   u32x4 rq[QT::PER_THREAD], rdo[QT::PER_THREAD];
-  float rstat = 0.f;  // threads 0..63: lse, 64..127: delta of the block's 64 queries
+  float rstat = 0.f;  // threads 0..63: -lse, 64..127: -delta of the block's 64 queries
 
   auto fetch = [&](int qb) {
     QT::fetch(rq, Q, p.ss, qb);
     QT::fetch(rdo, dO, p.ss, qb);
-    if (threadIdx.x < 64) rstat = lse[qb + threadIdx.x];
-    else if (threadIdx.x < 128) rstat = delta[qb + threadIdx.x - 64];
+    if (threadIdx.x < 64) rstat = -lse[qb + threadIdx.x];
+    else if (threadIdx.x < 128) rstat = -delta[qb + threadIdx.x - 64];
   };
   auto commit = [&](char* st) {
     QT::commit(st, rq);
@@ -360,42 +381,50 @@ __global__ __launch_bounds__(256) void attn_dkdv_kernel(AttnParams p) {
       for (int qt = 0; qt < 2; ++qt) {
         const int qs = qb + qt * 32;      // first query of this 32-row sub-tile
         if (qs + 31 < kw0) continue;      // entirely above the diagonal for this wave
-        const bool diag = qs < kw0 + 31;
-        f32x16 s, dp;
+        auto tile = [&](auto diag_tag) {
+          constexpr bool DIAG = decltype(diag_tag)::value;
+          // sstat holds -lse and -delta: dp starts at -delta, so dP - delta costs nothing
+          f32x16 s, dp;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
+          for (int g = 0; g < 4; ++g) {
+            const f32x4 d4 = *reinterpret_cast<const f32x4*>(sstat + 64 + qt * 32 + g * 8 + 4 * (lane >> 5));
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          s = mfma32(QT::frag_rows(sq, qt * 32, ks, lane), kf[ks], s);
-          dp = mfma32(QT::frag_rows(sdo, qt * 32, ks, lane), vf[ks], dp);
-        }
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const int ql = qt * 32 + g * 8 + 4 * (lane >> 5);  // block-local first query of the group
-          const f32x4 l4 = *reinterpret_cast<const f32x4*>(sstat + ql);
-          const f32x4 d4 = *reinterpret_cast<const f32x4*>(sstat + 64 + ql);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int qi = qb + ql + e;
-            float x = s[g * 4 + e] * p.scale_log2;
-            if (HAS_BIAS)
-              x += (float)((const T*)p.bias)[(int64_t)h * p.bias_sh + (int64_t)qi * p.bias_sr + mykey] * kLog2e;
-            float pr = fast_exp2(x - l4[e]);
-            if (diag && mykey > qi) pr = 0.f;
-            s[g * 4 + e] = pr;
-            dp[g * 4 + e] = pr * (dp[g * 4 + e] - d4[e]);
+            for (int e = 0; e < 4; ++e) { s[g * 4 + e] = 0.f; dp[g * 4 + e] = d4[e]; }
           }
-        }
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-          const v8 pa = round8<T>(s, t);
-          const v8 dsa = round8<T>(dp, t);
-#pragma unroll
-          for (int d = 0; d < DT; ++d) {
-            dv[d] = mfma32(QT::frag_hd(sdo, qt * 32 + t * 16, d, lane), pa, dv[d]);
-            dk[d] = mfma32(QT::frag_hd(sq, qt * 32 + t * 16, d, lane), dsa, dk[d]);
+          for (int ks = 0; ks < KS; ++ks) {
+            s = mfma32(QT::frag_rows(sq, qt * 32, ks, lane), kf[ks], s);
+            dp = mfma32(QT::frag_rows(sdo, qt * 32, ks, lane), vf[ks], dp);
           }
-        }
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const int ql = qt * 32 + g * 8 + 4 * (lane >> 5);  // block-local first query of the group
+            const f32x4 l4 = *reinterpret_cast<const f32x4*>(sstat + ql);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int qi = qb + ql + e;
+              float x = fmaf(s[g * 4 + e], p.scale_log2, l4[e]);  // s*scale*log2e - lse
+              if (HAS_BIAS)
+                x += (float)((const T*)p.bias)[(int64_t)h * p.bias_sh + (int64_t)qi * p.bias_sr + mykey] * kLog2e;
+              float pr = fast_exp2(x);
+              if (DIAG && mykey > qi) pr = 0.f;
+              s[g * 4 + e] = pr;
+              dp[g * 4 + e] *= pr;
+            }
+          }
+#pragma unroll
+          for (int t = 0; t < 2; ++t) {
+            const v8 pa = round8<T>(s, t);
+            const v8 dsa = round8<T>(dp, t);
+#pragma unroll
+            for (int d = 0; d < DT; ++d) {
+              dv[d] = mfma32(QT::frag_hd(sdo, qt * 32 + t * 16, d, lane), pa, dv[d]);
+              dk[d] = mfma32(QT::frag_hd(sq, qt * 32 + t * 16, d, lane), dsa, dk[d]);
+            }
+          }
+        };
+        if (qs < kw0 + 31) tile(std::true_type{});
+        else tile(std::false_type{});
       }
     }
     if (more) commit(smem + ((it + 1) & 1) * STAGE);
@@ -427,7 +456,7 @@ __global__ __launch_bounds__(256) void attn_dkdv_kernel(AttnParams p) {
 // diagonal, K and V tiles through LDS.
 // ===========================================================================
 template <typename T, int HD, bool HAS_BIAS>
-__global__ __launch_bounds__(256) void attn_dq_kernel(AttnParams p) {
+__global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_dq_kernel(AttnParams p) {
   typedef SeqTile<T, 64, HD> KT;
   typedef typename Vec<T>::v8 v8;
   typedef typename Vec<T>::v4 v4;
@@ -455,7 +484,7 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(AttnParams p) {
   const int nkv = kv_end / 64;
 
   v8 qf[KS], dof[KS];
-  float my_lse = 0.f, my_delta = 0.f;
+  float neg_lse = 0.f, neg_delta = 0.f;
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
     u32x4 a = {0u, 0u, 0u, 0u}, c = {0u, 0u, 0u, 0u};
@@ -467,8 +496,8 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(AttnParams p) {
     dof[ks] = __builtin_bit_cast(v8, c);
   }
   if (active) {
-    my_lse = p.lse[(int64_t)bh * p.S + myq];
-    my_delta = p.delta[(int64_t)bh * p.S + myq];
+    neg_lse = -p.lse[(int64_t)bh * p.S + myq];
+    neg_delta = -p.delta[(int64_t)bh * p.S + myq];
   }
   f32x16 dq[DT];
 #pragma unroll
@@ -497,38 +526,44 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(AttnParams p) {
       for (int jt = 0; jt < 2; ++jt) {
         const int ks0 = kb + jt * 32;  // first key of this 32-key sub-tile
         if (ks0 > q0w + 31) continue;
-        const bool diag = ks0 + 31 > q0w;
-        f32x16 s, dp;
+        auto tile = [&](auto diag_tag) {
+          constexpr bool DIAG = decltype(diag_tag)::value;
+          f32x16 s, dp;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
+          for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = neg_delta; }  // dP - delta for free
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          s = mfma32(KT::frag_rows(sk, jt * 32, ks, lane), qf[ks], s);
-          dp = mfma32(KT::frag_rows(sv, jt * 32, ks, lane), dof[ks], dp);
-        }
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const int key0 = ks0 + g * 8 + 4 * (lane >> 5);
-          float bv[4] = {0.f, 0.f, 0.f, 0.f};
-          if (HAS_BIAS) {
-            const v4 raw = *reinterpret_cast<const v4*>((const T*)p.bias + (int64_t)h * p.bias_sh +
-                                                        (int64_t)myq * p.bias_sr + key0);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) bv[e] = (float)raw[e] * kLog2e;
+          for (int ks = 0; ks < KS; ++ks) {
+            s = mfma32(KT::frag_rows(sk, jt * 32, ks, lane), qf[ks], s);
+            dp = mfma32(KT::frag_rows(sv, jt * 32, ks, lane), dof[ks], dp);
           }
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            float pr = fast_exp2(s[g * 4 + e] * p.scale_log2 + bv[e] - my_lse);
-            if (diag && key0 + e > myq) pr = 0.f;
-            dp[g * 4 + e] = pr * (dp[g * 4 + e] - my_delta);
+          for (int g = 0; g < 4; ++g) {
+            const int key0 = ks0 + g * 8 + 4 * (lane >> 5);
+            float bv[4] = {0.f, 0.f, 0.f, 0.f};
+            if (HAS_BIAS) {
+              const v4 raw = *reinterpret_cast<const v4*>((const T*)p.bias + (int64_t)h * p.bias_sh +
+                                                          (int64_t)myq * p.bias_sr + key0);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) bv[e] = (float)raw[e] * kLog2e;
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              float x = fmaf(s[g * 4 + e], p.scale_log2, neg_lse);
+              if (HAS_BIAS) x += bv[e];
+              float pr = fast_exp2(x);
+              if (DIAG && key0 + e > myq) pr = 0.f;
+              dp[g * 4 + e] *= pr;
+            }
           }
-        }
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-          const v8 dsb = round8<T>(dp, t);
+          for (int t = 0; t < 2; ++t) {
+            const v8 dsb = round8<T>(dp, t);
 #pragma unroll
-          for (int d = 0; d < DT; ++d) dq[d] = mfma32(KT::frag_hd(sk, jt * 32 + t * 16, d, lane), dsb, dq[d]);
-        }
+            for (int d = 0; d < DT; ++d) dq[d] = mfma32(KT::frag_hd(sk, jt * 32 + t * 16, d, lane), dsb, dq[d]);
+          }
+        };
+        if (ks0 + 31 > q0w) tile(std::true_type{});
+        else tile(std::false_type{});
       }
     }
     if (more) {
