@@ -1,0 +1,111 @@
+"""C-ABI library: loads, exports every symbol include/tritonformer_amd.h declares,
+and rejects bad arguments on the host before anything is launched (so these run
+without a GPU).  Mirrors the reference's Python asserts (kernels/gemm.py:370-377,
+kernels/attention.py:181-183, 567-570, kernels/biased_attention.py:199-207,
+kernels/layernorm.py:68-71) as status codes."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from tritonformer_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "tritonformer_amd.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(tf_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_surface():
+    names = declared_functions()
+    for must in ["tf_gemm", "tf_attn_fwd", "tf_attn_bwd", "tf_layernorm_fwd", "tf_layernorm_bwd", "tf_softmax_fwd",
+                 "tf_softmax_bwd", "tf_cross_entropy_fwd", "tf_cross_entropy_bwd", "tf_colsum", "tf_relu_mask",
+                 "tf_status_string", "tf_version"]:
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared_functions():
+        assert hasattr(lib, name), f"{name} declared in the header but not exported"
+
+
+def test_binding_table_matches_header():
+    assert sorted(_lib.SIGNATURES) == declared_functions()
+
+
+def test_status_strings():
+    lib = _lib.load()
+    assert lib.tf_version() >= 100
+    assert lib.tf_status_string(0) == b"ok"
+    for code in range(-6, 0):
+        assert len(lib.tf_status_string(code)) > 3
+
+
+FAKE = 0x1000  # non-null, 16-byte aligned; never dereferenced because the checks fail first
+
+
+def test_gemm_rejects_bad_arguments():
+    lib = _lib.load()
+    g = lib.tf_gemm
+    ok_tail = (FAKE, 64, FAKE, 64, FAKE, 64, None, 0, None, 0)
+    assert g(None, 0, 0, 1, 64, 64, 64, None, 64, FAKE, 64, FAKE, 64, None, 0, None, 0) == -1   # null A
+    assert g(None, 0, 0, 1, 0, 64, 64, *ok_tail) == -1                                          # M = 0
+    assert g(None, 2, 0, 1, 64, 64, 64, *ok_tail) == -2                                         # fp32 operands
+    assert g(None, 0, 5, 1, 64, 64, 64, *ok_tail) == -1                                         # bad layout
+    assert g(None, 0, 0, 1, 64, 64, 64, FAKE, 32, FAKE, 64, FAKE, 64, None, 0, None, 0) == -4   # lda < K
+    assert g(None, 0, 0, 1, 64, 64, 64, FAKE + 1, 64, FAKE, 64, FAKE, 64, None, 0, None, 0) == -3  # odd pointer
+    # a split contraction without workspace is refused, and the size query says how much is needed
+    need = lib.tf_gemm_workspace_bytes(1, 1, 1024, 1024, 8192)
+    assert need > 0 and need % (1024 * 1024 * 4) == 0
+    assert g(None, 0, 1, 1, 1024, 1024, 8192, FAKE, 1024, FAKE, 1024, FAKE, 1024, None, 0, None, 0) == -5
+    assert lib.tf_gemm_workspace_bytes(0, 1, 8192, 4096, 1024) == 0
+    assert lib.tf_gemm_out(None, 0, 1, 0, 1, 64, 64, 64, *ok_tail) == -2                        # bf16 out of fp16 in
+
+
+def test_attention_rejects_bad_shapes():
+    lib = _lib.load()
+
+    def fwd(S, hd, ss=None, dtype=0, bias=None, bsr=0):
+        ss = ss if ss is not None else hd
+        return lib.tf_attn_fwd(None, dtype, 1, 2, S, hd, FAKE, FAKE, FAKE, FAKE, S * 2 * hd, hd, 2 * hd if ss == hd else ss,
+                               FAKE, bias, bsr * bsr if bias else 0, bsr, 0.125)
+
+    assert fwd(100, 64) == -4           # S % 64 != 0
+    assert fwd(128, 48) == -4           # head_dim not in {32, 64, 128}
+    assert fwd(128, 64, dtype=2) == -2  # fp32
+    assert fwd(128, 64, ss=60) == -3    # row stride not a multiple of 8 elements
+    assert fwd(128, 64, bias=FAKE, bsr=64) == -3   # bias rows shorter than S
+    assert lib.tf_attn_bwd(None, 0, 1, 2, 128, 64, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, None, 16384, 64, 128,
+                           FAKE, FAKE, None, 0, 0, 0.125) == -1  # null dv
+
+
+def test_row_kernels_reject_bad_arguments():
+    lib = _lib.load()
+    assert lib.tf_layernorm_fwd(None, 2, 4, 64, FAKE, 64, FAKE, FAKE, 1e-5, FAKE, 64, FAKE, FAKE) == -2
+    assert lib.tf_layernorm_fwd(None, 0, 4, 64, FAKE, 32, FAKE, FAKE, 1e-5, FAKE, 64, FAKE, FAKE) == -1
+    assert lib.tf_layernorm_bwd(None, 0, 4, 64, FAKE, 64, FAKE, 64, FAKE, FAKE, FAKE, FAKE, 64, FAKE, FAKE,
+                                None, 0) == -5
+    assert lib.tf_layernorm_bwd_partial_bytes(8192, 1024) == 512 * 2 * 1024 * 4
+    assert lib.tf_softmax_fwd(None, 0, 4, 0, FAKE, 64, FAKE, 64) == -1
+    assert lib.tf_cross_entropy_fwd(None, 2, 4, 64, FAKE, 64, FAKE, FAKE, FAKE) == -2
+    assert lib.tf_cross_entropy_bwd(None, 0, 4, 64, FAKE, 32, FAKE, FAKE, FAKE, 1, FAKE, 64) == -1
+    assert lib.tf_colsum(None, 0, 16, 64, FAKE, 64, FAKE, None, 0) == -5
+    assert lib.tf_relu_mask(None, 0, 4, 64, None, 64, FAKE, 64, FAKE, 64) == -1
+    # empty inputs are accepted and launch nothing
+    assert lib.tf_softmax_fwd(None, 0, 0, 64, FAKE, 64, FAKE, 64) == 0
+    assert lib.tf_cross_entropy_fwd(None, 0, 0, 64, FAKE, 64, FAKE, FAKE, FAKE) == 0
+    assert lib.tf_relu_mask(None, 0, 0, 64, FAKE, 64, FAKE, 64, FAKE, 64) == 0
+
+
+def test_check_maps_status_to_exceptions():
+    with pytest.raises(ValueError):
+        _lib.check(-4)
+    with pytest.raises(_lib.TritonformerAmdError):
+        _lib.check(-5)
+    _lib.check(0)

@@ -1,0 +1,126 @@
+"""GPU parity of causal flash attention (forward, dQ, dK, dV) against the fp32
+oracle; mirrors the reference's tritonformer/test_attention.py (q, k, v, dy ~
+N(0,1) fp16; B in [1,4), nh in [4,32), S = 64*[1,32), hd in {32,64}) and adds
+hd = 128, bf16, the strided (B,S,nh,hd)->(B,nh,S,hd) views the model feeds, and
+the baseline configurations' shapes.
+
+Tolerance: max-abs <= 1e-2 (+1e-3 relative), as test_attention.py:88 (atol=1e-2),
+against fp32 math instead of the reference's fp16-rounded P.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import tritonformer_amd as T
+from oracle import ref_torch as R
+from tests.util import NUM_TEST, assert_close
+
+pytestmark = pytest.mark.gpu
+rng = np.random.RandomState(0)
+
+DIMS = [(int(b), int(nh), int(sq), int(hd))
+        for b in rng.randint(1, 4, size=NUM_TEST)
+        for nh in rng.randint(4, 12, size=1)
+        for sq in 64 * rng.randint(1, 12, size=NUM_TEST)
+        for hd in rng.choice([32, 64], size=1)]
+EDGE = [(1, 1, 64, 64), (1, 2, 64, 32), (2, 3, 128, 64), (1, 2, 192, 128), (1, 4, 320, 128), (2, 2, 1024, 64)]
+
+
+def make_qkv(dims, dtype, dev, seed=0, strided=True):
+    b, nh, s, hd = dims
+    g = torch.Generator().manual_seed(seed)
+    if strided:  # views of (B, S, nh*hd) buffers, strides (S*d, hd, d, 1), as transformer.py:158-175
+        raw = [torch.randn(b, s, nh * hd, generator=g).to(dtype) for _ in range(4)]
+        q, k, v, do = (t.view(b, s, nh, hd).permute(0, 2, 1, 3) for t in raw)
+    else:
+        q, k, v, do = (torch.randn(b, nh, s, hd, generator=g).to(dtype) for _ in range(4))
+    return q, k, v, do
+
+
+def run_case(dims, dtype, dev, bias=None, strided=True, seed=0):
+    q, k, v, do = make_qkv(dims, dtype, dev, seed, strided)
+    qd, kd, vd = (t.to(dev).requires_grad_(True) for t in (q, k, v))  # .to keeps the strides
+    if bias is None:
+        o = T.fast_causal_attention.apply(qd, kd, vd)
+    else:
+        o = T.fast_causal_attention_with_bias.apply(qd, kd, vd, bias.to(dev))
+    assert o.stride() == qd.stride() and o.dtype == dtype
+    o.backward(do.to(dev))
+    qr, kr, vr = (t.float().requires_grad_(True) for t in (q, k, v))
+    o_ref = R.causal_attention(qr, kr, vr, bias)
+    o_ref.backward(do.float())
+    tag = f"{dims} {dtype}"
+    assert_close(o, o_ref, dtype, "o " + tag)
+    assert_close(qd.grad, qr.grad, dtype, "dq " + tag)
+    assert_close(kd.grad, kr.grad, dtype, "dk " + tag)
+    assert_close(vd.grad, vr.grad, dtype, "dv " + tag)
+    return o, qd, kd, vd
+
+
+@pytest.mark.parametrize("dims", DIMS + EDGE)
+def test_attn_fwd_bwd(dims, dev):
+    run_case(dims, torch.float16, dev)
+
+
+@pytest.mark.parametrize("dims", [(1, 2, 128, 64), (2, 3, 256, 32), (1, 2, 192, 128)])
+def test_attn_bf16(dims, dev):
+    run_case(dims, torch.bfloat16, dev)
+
+
+def test_attn_contiguous_layout(dev):
+    run_case((2, 4, 256, 64), torch.float16, dev, strided=False)
+
+
+def test_attn_mismatched_strides_are_normalised(dev):
+    """The reference silently uses q's strides for k, v and o (kernels/attention.py:202-205)."""
+    q, k, v, do = make_qkv((1, 2, 128, 64), torch.float16, dev, strided=True)
+    kc = k.contiguous()
+    o = T.fast_causal_attention.apply(q.to(dev), kc.to(dev), v.to(dev))
+    assert_close(o, R.causal_attention(q, k, v), name="mixed layouts")
+
+
+def test_attn_invariants(dev):
+    o, q, k, v = run_case((2, 4, 512, 64), torch.float16, dev, seed=7)
+    assert torch.equal(o[:, :, 0], v.detach()[:, :, 0])        # query 0 attends to key 0 only
+    # a constant V makes every output row that constant, and dQ = dK = 0
+    vc = torch.ones_like(v.detach()) * 0.5
+    qd, kd = q.detach().clone().requires_grad_(True), k.detach().clone().requires_grad_(True)
+    oc = T.fast_causal_attention.apply(qd, kd, vc)
+    assert (oc.float() - 0.5).abs().max() < 2e-3
+    oc.backward(torch.randn_like(oc))
+    assert qd.grad.abs().max() < 2e-3 and kd.grad.abs().max() < 2e-3
+    # bitwise reproducible
+    assert torch.equal(T.fast_causal_attention.apply(q, k, v), o)
+
+
+def test_attn_large_magnitude_scores(dev):
+    """Scores far from zero exercise the thresholded running-max update."""
+    q, k, v, do = make_qkv((1, 2, 256, 64), torch.float16, dev, seed=3)
+    q = q * 6.0
+    o = T.fast_causal_attention.apply(q.to(dev), k.to(dev), v.to(dev))
+    assert_close(o, R.causal_attention(q, k, v), name="peaked softmax")
+
+
+@pytest.mark.parametrize("dims", [(4, 16, 2048, 64), (2, 16, 2048, 128)])
+def test_baseline_config_shapes(dims, dev):
+    """410M (hd 64) and 1.4B (hd 128) attention shapes at full size; oracle in fp32 on the GPU."""
+    b, nh, s, hd = dims
+    g = torch.Generator().manual_seed(0)
+    raw = [torch.randn(b, s, nh * hd, generator=g).half().to(dev) for _ in range(4)]
+    q, k, v, do = (t.view(b, s, nh, hd).permute(0, 2, 1, 3) for t in raw)
+    q, k, v = (t.requires_grad_(True) for t in (q, k, v))
+    o = T.fast_causal_attention.apply(q, k, v)
+    o.backward(do)
+    grads = [t.grad.clone() for t in (q, k, v)]
+    for t in (q, k, v):
+        t.grad = None
+    worst = 0.0
+    for bi in range(b):  # per batch element: keeps the S x S fp32 score matrix small
+        qr, kr, vr = (t[bi:bi + 1].detach().float().requires_grad_(True) for t in (q, k, v))
+        orf = R.causal_attention(qr, kr, vr)
+        orf.backward(do[bi:bi + 1].float())
+        assert_close(o[bi:bi + 1], orf, name="o")
+        for got, ref, nm in zip(grads, (qr, kr, vr), "qkv"):
+            assert_close(got[bi:bi + 1], ref.grad, name="d" + nm)

@@ -1,0 +1,78 @@
+"""GPU parity of the cross-entropy Function against the fp32 oracle.  The
+contract is the one the model uses (reference transformer.py:336-343): a loss
+per row, mean taken by the caller; reference test shapes N in [1,32), V in
+[256,64000) (tritonformer/test_crossentropy.py).  Tolerance: loss atol 1e-2 as
+the reference's test; gradient atol 1e-3 on probabilities in [0,1]."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import tritonformer_amd as T
+from oracle import ref_torch as R
+from tests.util import NUM_TEST, assert_close, rel_l2
+
+pytestmark = pytest.mark.gpu
+rng = np.random.RandomState(0)
+DIMS = [(int(n), int(v)) for n in rng.randint(1, 32, size=NUM_TEST) for v in rng.randint(256, 64000, size=NUM_TEST)]
+EDGE = [(1, 8), (3, 7), (5, 50304), (64, 50304), (2, 131072)]
+
+
+@pytest.mark.parametrize("dims", DIMS + EDGE)
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_cross_entropy_fwd_bwd(dims, dtype, dev):
+    n, v = dims
+    g = torch.Generator().manual_seed(n + v)
+    x = torch.randn(n, v, generator=g).to(dtype)
+    lab = torch.randint(0, v, (n,), generator=g)
+    gout = torch.randn(n, generator=g).to(dtype)
+    xd = x.to(dev).requires_grad_(True)
+    loss = T.cross_entropy_loss.apply(xd, lab.to(dev))
+    assert loss.shape == (n,) and loss.dtype == dtype
+    loss.backward(gout.to(dev))
+    assert_close(loss, R.cross_entropy(x, lab), dtype, f"loss {dims}", atol=1e-2 if dtype == torch.float16 else 6e-2)
+    assert_close(xd.grad, R.cross_entropy_bwd(x, lab, gout), dtype, f"grad {dims}", atol=1e-3, rtol=1e-2)
+
+
+def test_uniform_logits_and_mean_reduction(dev):
+    n, v = 16, 50304
+    x = torch.zeros(n, v, dtype=torch.float16, device=dev, requires_grad=True)
+    lab = torch.randint(0, v, (n,), device=dev)
+    loss = T.cross_entropy_loss.apply(x, lab)
+    assert (loss.float() - math.log(v)).abs().max() < 5e-3          # ln(50304) = 10.8258
+    loss.float().mean().backward()                                   # the caller's reduction
+    grad = x.grad.float()
+    assert (grad.sum(-1)).abs().max() < 1e-3                         # softmax - onehot sums to zero
+    assert torch.equal(grad.argmin(-1), lab)
+
+
+def test_row_stride_and_labels_edge(dev):
+    """Logits that are a column slice of a wider buffer (row stride > V) and labels at both ends."""
+    g = torch.Generator().manual_seed(3)
+    wide = torch.randn(9, 1000, generator=g).half()
+    x = wide[:, :904]
+    lab = torch.tensor([0, 903, 5, 17, 903, 0, 450, 1, 902])
+    loss = T.cross_entropy_loss.apply(x.to(dev), lab.to(dev))
+    assert_close(loss, R.cross_entropy(x, lab), name="strided rows")
+
+
+def test_headline_rows(dev):
+    """Rows of the 410M configuration (V = 50304) with unit-variance logits; fp32 oracle on the GPU."""
+    n, v = 2047, 50304
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(n, v, generator=g).half().to(dev).requires_grad_(True)
+    lab = torch.randint(0, v, (n,), generator=g).to(dev)
+    loss = T.cross_entropy_loss.apply(x, lab)
+    loss.float().sum().backward()
+    ref = R.cross_entropy(x.detach(), lab)
+    assert_close(loss, ref, name="loss")
+    assert abs(loss.float().mean().item() - ref.mean().item()) <= 1e-3 * ref.mean().item()
+    assert rel_l2(x.grad, R.cross_entropy_bwd(x.detach(), lab, torch.ones(n, device=dev))) < 2e-3
+
+
+def test_argument_checks(dev):
+    with pytest.raises(TypeError):
+        T.cross_entropy_loss.apply(torch.zeros(4, 8, device=dev, dtype=torch.float16), torch.zeros(4, device=dev, dtype=torch.int32))
+    with pytest.raises(ValueError):
+        T.cross_entropy_loss.apply(torch.zeros(4, 8, device=dev, dtype=torch.float16), torch.zeros(5, device=dev, dtype=torch.int64))

@@ -1,0 +1,179 @@
+"""GPU parity of the four Linear Functions against the fp32 oracle; mirrors the
+reference's tritonformer/test_linear.py (random shapes that are not tile
+multiples, x ~ N(0,1), W ~ N(0,1)/sqrt(in), dy ~ N(0,1)) and adds the ReLU
+variants, bf16 and the baseline configurations' exact shapes, which the
+reference does not test.
+
+Tolerance (fp16): |err| <= 1e-2 + 1e-3*|ref| per element (the reference uses
+atol 1e-2 against an fp16 result; the relative term is one fp16 rounding of the
+fp32 reference); bias gradient: relative L2 < 1e-3, as test_linear.py:28-30,169.
+"""
+import numpy as np
+import pytest
+import torch
+
+import tritonformer_amd as T
+from oracle import ref_torch as R
+from tests.util import NUM_TEST, assert_close, rel_l2
+
+pytestmark = pytest.mark.gpu
+rng = np.random.RandomState(0)
+
+RANDOM_DIMS = [(int(b), int(m), int(n), int(k))
+               for b in rng.randint(1, 8, size=NUM_TEST)
+               for m in rng.randint(64, 1024, size=1)
+               for n in rng.randint(64, 1536, size=NUM_TEST)
+               for k in rng.randint(64, 1536, size=1)]
+EDGE_DIMS = [(1, 1, 8, 8), (1, 64, 64, 64), (2, 77, 333, 129), (3, 130, 264, 520), (1, 257, 1024, 72),
+             (2, 512, 768, 3072), (1, 300, 4096, 1024)]
+VARIANTS = {
+    "nobias": (T.linear_no_bias, False, False),
+    "bias": (T.linear_bias, True, False),
+    "relu": (T.linear_fused_relu, False, True),
+    "biasrelu": (T.linear_fused_bias_relu, True, True),
+}
+
+
+def make(dims, dtype, dev, seed):
+    b, m, n, k = dims
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(b, m, n, generator=g).to(dtype)
+    w = (torch.randn(n, k, generator=g) / n ** 0.5).to(dtype)
+    bias = torch.randn(k, generator=g).to(dtype)
+    dy = torch.randn(b, m, k, generator=g).to(dtype)
+    return x, w, bias, dy
+
+
+def run_case(dims, variant, dtype, dev, seed=0):
+    fn, use_bias, relu = VARIANTS[variant]
+    x, w, bias, dy = make(dims, dtype, dev, seed)
+    xd, wd, bd = (t.to(dev).requires_grad_(True) for t in (x, w, bias))
+    y = fn.apply(xd, wd, bd) if use_bias else fn.apply(xd, wd)
+    y.backward(dy.to(dev))
+    y_ref = R.linear(x, w, bias if use_bias else None, relu)
+    assert_close(y, y_ref, dtype, f"{variant} y {dims}")
+    # the ReLU gradient mask is the sign of the kernel's own rounded output (as in the
+    # reference, linear.py:62): on a pre-activation within rounding of zero fp32 and
+    # 16-bit math may disagree, which is not an error of the backward kernels
+    act = y.detach().cpu() if relu else None
+    dx_ref, dw_ref, db_ref = R.linear_bwd(x, w, dy, act=act, with_bias=use_bias)
+    big = dims[0] * dims[1]  # contraction length of dW: rounding noise grows like sqrt
+    assert_close(xd.grad, dx_ref, dtype, f"{variant} dx {dims}")
+    assert_close(wd.grad, dw_ref, dtype, f"{variant} dw {dims}", atol=1e-2 * max(1.0, (big / 512) ** 0.5) * (6 if dtype == torch.bfloat16 else 1))
+    assert wd.grad.shape == w.shape
+    if use_bias:
+        assert bd.grad.shape == bias.shape
+        assert rel_l2(bd.grad, db_ref) < (1e-3 if dtype == torch.float16 else 8e-3), f"{variant} db {dims}"
+
+
+@pytest.mark.parametrize("dims", RANDOM_DIMS + EDGE_DIMS)
+@pytest.mark.parametrize("variant", ["nobias", "bias"])
+def test_linear_fwd_bwd(dims, variant, dev):
+    run_case(dims, variant, torch.float16, dev)
+
+
+@pytest.mark.parametrize("dims", EDGE_DIMS + RANDOM_DIMS[:3])
+@pytest.mark.parametrize("variant", ["relu", "biasrelu"])
+def test_linear_relu_fwd_bwd(dims, variant, dev):
+    run_case(dims, variant, torch.float16, dev)
+
+
+@pytest.mark.parametrize("dims", [(2, 77, 333, 129), (2, 256, 1024, 512)])
+@pytest.mark.parametrize("variant", list(VARIANTS))
+def test_linear_bf16(dims, variant, dev):
+    run_case(dims, variant, torch.bfloat16, dev)
+
+
+def test_relu_fused_equals_unfused(dev):
+    x, w, bias, _ = make((2, 100, 256, 384), torch.float16, dev, 3)
+    xd, wd, bd = x.to(dev), w.to(dev), bias.to(dev)
+    assert torch.equal(T.linear_fused_relu.apply(xd, wd), torch.relu(T.linear_no_bias.apply(xd, wd)))
+    assert torch.equal(T.linear_fused_bias_relu.apply(xd, wd, bd), torch.relu(T.linear_bias.apply(xd, wd, bd)))
+
+
+def test_identity_and_permutation_weights(dev):
+    x = torch.randn(2, 70, 128).half().to(dev)
+    eye = torch.eye(128).half().to(dev)
+    assert torch.equal(T.linear_no_bias.apply(x, eye), x)
+    perm = torch.randperm(128)
+    assert torch.equal(T.linear_no_bias.apply(x, eye[:, perm.to(dev)]), x[..., perm.to(dev)])
+
+
+def test_grad_buffers_not_mutated_and_deterministic(dev):
+    """The reference masks grad_output in place (kernels/activation.py:24); ours must
+    leave autograd's buffer alone, and two runs must agree bit for bit."""
+    x, w, bias, dy = make((2, 128, 256, 512), torch.float16, dev, 5)
+    xd, wd = x.to(dev).requires_grad_(True), w.to(dev).requires_grad_(True)
+    dyd = dy.to(dev)
+    keep = dyd.clone()
+    y = T.linear_fused_relu.apply(xd, wd)
+    y.backward(dyd, retain_graph=True)
+    g1 = (xd.grad.clone(), wd.grad.clone())
+    assert torch.equal(dyd, keep)
+    xd.grad = wd.grad = None
+    y.backward(dyd)
+    assert torch.equal(g1[0], xd.grad) and torch.equal(g1[1], wd.grad)
+
+
+def test_transposed_weight_view_and_noncontiguous_input(dev):
+    x = torch.randn(2, 96, 160).half()
+    w = torch.randn(200, 160).half() / 12.0
+    y = T.linear_no_bias.apply(x.to(dev), w.to(dev).T)          # stride-(1, K) view, as linear.py:23 passes
+    assert_close(y, R.linear(x, w.T), name="transposed weight")
+    xt = torch.randn(2, 160, 96).half()
+    y2 = T.linear_no_bias.apply(xt.to(dev).transpose(1, 2), w.to(dev).T)
+    assert_close(y2, R.linear(xt.transpose(1, 2), w.T), name="non-contiguous input")
+
+
+def test_autocast_fp32_master_weights(dev):
+    """custom_fwd(cast_inputs=float16) semantics (reference linear.py:14): fp32 inputs are
+    cast inside autocast; gradients come back in fp32."""
+    x = torch.randn(2, 64, 128, device=dev, requires_grad=True)
+    w = (torch.randn(128, 256, device=dev) / 11.3).requires_grad_(True)
+    b = torch.randn(256, device=dev, requires_grad=True)
+    with torch.autocast("cuda", dtype=torch.float16):
+        y = T.linear_bias.apply(x, w, b)
+    assert y.dtype == torch.float16
+    y.float().sum().backward()
+    assert x.grad.dtype == w.grad.dtype == b.grad.dtype == torch.float32
+    dx, dw, db = R.linear_bwd(x.detach().cpu(), w.detach().cpu(), torch.ones(2, 64, 256), with_bias=True)
+    assert rel_l2(w.grad, dw) < 2e-3 and rel_l2(x.grad, dx) < 2e-3 and rel_l2(b.grad, db) < 1e-3
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        assert T.linear_no_bias.apply(x, w).dtype == torch.bfloat16
+    with pytest.raises(TypeError):   # outside autocast fp32 inputs are not accepted (16-bit kernels only)
+        T.linear_no_bias.apply(x, w)
+
+
+@pytest.mark.parametrize("shape", [(4, 2048, 1024, 4096), (4, 2048, 4096, 1024), (4, 2048, 1024, 1024)])
+def test_headline_config_shapes(shape, dev):
+    """410M / ctx 2048 / bs 4 layer shapes at full size; the oracle runs in fp32 on
+    the GPU here (same expressions, rocBLAS fp32) to keep the CPU time bounded."""
+    b, s, n, k = shape
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(b, s, n, generator=g).half().to(dev).requires_grad_(True)
+    w = (torch.randn(n, k, generator=g) * 0.02).half().to(dev).requires_grad_(True)
+    dy = torch.randn(b, s, k, generator=g).half().to(dev)
+    y = T.linear_no_bias.apply(x, w)
+    y.backward(dy)
+    assert_close(y, R.linear(x.detach(), w.detach()), name="y")
+    dx, dw, _ = R.linear_bwd(x.detach(), w.detach(), dy)
+    assert_close(x.grad, dx, name="dx")
+    assert rel_l2(w.grad, dw) < 1e-3
+    # linearity in dy: the weight gradient of 2*dy is exactly twice (power-of-two scaling is exact in fp16)
+    x.grad = w.grad = None
+    T.linear_no_bias.apply(x, w).backward(2 * dy)
+    assert rel_l2(w.grad, 2 * dw) < 1e-3
+
+
+def test_logits_projection_shape(dev):
+    """hidden -> vocab projection of the headline model on a slice of the tokens."""
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(1, 512, 1024, generator=g).half().to(dev).requires_grad_(True)
+    w = (torch.randn(1024, 50304, generator=g) * 0.02).half().to(dev).requires_grad_(True)
+    y = T.linear_no_bias.apply(x, w)
+    dy = (torch.randn(1, 512, 50304, generator=g) * 0.1).half().to(dev)
+    y.backward(dy)
+    assert_close(y, R.linear(x.detach(), w.detach()), name="logits")
+    dx, dw, _ = R.linear_bwd(x.detach(), w.detach(), dy)
+    assert_close(x.grad, dx, name="dx", atol=2e-2)
+    assert rel_l2(w.grad, dw) < 1e-3

@@ -1,0 +1,48 @@
+"""GPU parity of the Softmax Function against the fp32 oracle; mirrors the
+reference's tritonformer/test_softmax.py (fp32 input, dy = 0.1*randn, atol 1e-4)
+and adds the 16-bit dtypes."""
+import numpy as np
+import pytest
+import torch
+
+import tritonformer_amd as T
+from oracle import ref_torch as R
+from tests.util import NUM_TEST, assert_close
+
+pytestmark = pytest.mark.gpu
+rng = np.random.RandomState(0)
+DIMS = [(int(b), int(r), int(c)) for b in rng.randint(1, 8, size=NUM_TEST) for r in rng.randint(256, 512, size=1)
+        for c in rng.randint(64, 1024, size=NUM_TEST)]
+EDGE = [(1, 1, 1), (1, 3, 5), (2, 64, 1024), (1, 17, 2048), (1, 9, 2052), (1, 4, 9000)]
+
+
+@pytest.mark.parametrize("dims", DIMS + EDGE)
+def test_softmax_fp32_fwd_bwd(dims, dev):
+    g = torch.Generator().manual_seed(sum(dims))
+    x = torch.randn(*dims, generator=g)
+    dy = 0.1 * torch.randn(*dims, generator=g)
+    xd = x.to(dev).requires_grad_(True)
+    y = T.Softmax.apply(xd)
+    assert y.dtype == torch.float32          # dtype preserved, no autocast hook (reference softmax.py:9-10)
+    y.backward(dy.to(dev))
+    y_ref = R.softmax(x)
+    assert_close(y, y_ref, torch.float32, f"y {dims}")          # atol 1e-4 as test_softmax.py:44
+    assert_close(xd.grad, R.softmax_bwd(y_ref, dy), torch.float32, f"dx {dims}")
+    assert (y.sum(-1) - 1).abs().max() < 1e-5
+    assert xd.grad.sum(-1).abs().max() < 1e-5
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("dims", [(2, 100, 777), (3, 64, 1024)])
+def test_softmax_16bit(dims, dtype, dev):
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(*dims, generator=g).to(dtype)
+    dy = (0.1 * torch.randn(*dims, generator=g)).to(dtype)
+    xd = x.to(dev).requires_grad_(True)
+    y = T.Softmax.apply(xd)
+    keep = dy.to(dev)
+    before = keep.clone()
+    y.backward(keep)
+    assert torch.equal(keep, before)          # grad_out is not overwritten (the reference does, softmax.py:101-111)
+    assert_close(y, R.softmax(x), dtype, "y", atol=2e-3)
+    assert_close(xd.grad, R.softmax_bwd(y.detach().cpu(), dy), dtype, "dx", atol=2e-3)

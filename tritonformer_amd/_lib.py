@@ -71,6 +71,8 @@ def check(status):
         msg = load().tf_status_string(status).decode()
         if status in (-1, -3, -4):
             raise ValueError(f"tritonformer_amd: {msg}")
+        if status == -2:
+            raise TypeError(f"tritonformer_amd: {msg}")
         raise TritonformerAmdError(f"tritonformer_amd: {msg}")
 
 

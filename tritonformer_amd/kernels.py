@@ -43,6 +43,8 @@ def _check_linear(a, b, bias=None):
         raise ValueError("Incorrect number of dimensions for LHS or RHS")
     if a.shape[2] != b.shape[0]:
         raise ValueError("Inner dimensions of the two operands do not match")
+    if a.dtype not in (torch.float16, torch.bfloat16):
+        raise TypeError("linear kernels take float16 or bfloat16 operands (use autocast for fp32 parameters)")
     if a.dtype != b.dtype or (bias is not None and bias.dtype != a.dtype):
         raise TypeError("operands must share one 16-bit dtype")
     if bias is not None and (bias.ndim != 1 or bias.shape[0] != b.shape[1]):

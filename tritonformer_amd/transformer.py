@@ -41,7 +41,7 @@ def get_slopes(n: int) -> List[float]:
     power of two below n followed by every other slope of the next power."""
     def power_of_two(m):
         base = 2.0 ** (-(2.0 ** -(math.log2(m) - 3)))
-        return [base ** (i + 1) for i in range(m)]
+        return [base * base ** i for i in range(m)]  # same operation order as the reference: bit-identical slopes
 
     if n & (n - 1) == 0:
         return power_of_two(n)
