@@ -27,6 +27,9 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA
 PEAK_HBM_GBS = 8000.0
+# HBM bytes per GEMM launch at the headline workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# scaled against a copy kernel of known size (profiles/gemm_hbm_traffic_410m_step.md)
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = {"gpt2-410m-ctx2048-bs4": 104.4e6}
 
 WORKLOADS = {
     # name: (layers, d, heads, head_dim, ffn, seq, batch, linear_bias, alibi)
@@ -150,6 +153,9 @@ def main():
     ap.add_argument("--dtype", default="fp16", choices=["fp16", "bf16"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-roofline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain 1 GiB device-to-device copy kernel (known traffic: 1 GiB read, "
+                         "1 GiB written) so that rocprofv3 FETCH_SIZE / WRITE_SIZE readings can be scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported "
@@ -191,7 +197,7 @@ def main():
         "pct_of_fp16_mfma_peak": round(100.0 * tflops / PEAK_FP16_TFLOPS, 2),
         "tokens_per_s": round(B * S / (ms * 1e-3), 1),
         "step_tflop": round(flops / 1e12, 3),
-        "loss": round(float(loss), 4),
+        "loss": round(float(loss.detach()), 4),
     }
 
     if not args.no_roofline:
@@ -209,7 +215,7 @@ def main():
             "peak": PEAK_FP16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(achieved / PEAK_FP16_TFLOPS, 4),
-            "traffic": None,
+            "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload),
             "launches_per_step": launches // reps,
             "flop_per_launch": round(gflops / launches, 1),
             "avg_launch_us": round(total_ms / launches * 1e3, 2),
@@ -217,6 +223,11 @@ def main():
             "measured": f"HIP events on the launch stream around each tf_gemm call, {reps} instrumented steps "
                         "run after the timed ones (split-contraction launches include their reduce kernel)",
         }
+    if args.calibrate_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=device).normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.workload)
     print(json.dumps(out))
