@@ -55,8 +55,8 @@ struct Panel {
 
   // chunk-index swizzle; an involution on c for a fixed LDS row
   static __device__ __forceinline__ int swz(int lrow, int c) {
-    if (KMAJOR) return c ^ ((lrow / (16 / CPR)) % CPR);
-    return c ^ ((lrow & 3) << 2);
+    if constexpr (KMAJOR) return c ^ ((lrow / (16 / CPR)) % CPR);
+    else return c ^ ((lrow & 3) << 2);
   }
 
   // Global -> registers.  (row0, rmax) bound the m/n index, (k0, kend) the contraction.
@@ -283,6 +283,32 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_kernel(GemmParams p) {
 // ---------------------------------------------------------------------------
 typedef __attribute__((address_space(1))) const void gptr_void;
 
+// s_waitcnt lgkmcnt(n): at most n LDS reads (the youngest) may still be in flight.
+template <int N> __device__ __forceinline__ void wait_lgkmcnt() {
+  __builtin_amdgcn_s_waitcnt(15 | (3 << 14) | (7 << 4) | ((N & 15) << 8));
+}
+
+// LDS operand reads issued as volatile asm: the compiler neither reorders them nor
+// waits for them, so the kernel decides how far ahead of their MFMAs they run
+// (every consumer sits behind an explicit wait_lgkmcnt + scheduling barrier).
+__device__ __forceinline__ uint32_t lds_address(const char* p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
+}
+template <bool KMAJOR> struct FragRegs;
+template <> struct FragRegs<true> {
+  u32x4 q;
+  template <typename V8> __device__ __forceinline__ V8 get() const { return __builtin_bit_cast(V8, q); }
+};
+template <> struct FragRegs<false> {
+  u32x2 lo, hi;
+  template <typename V8> __device__ __forceinline__ V8 get() const {
+    const u32x4 v = {lo[0], lo[1], hi[0], hi[1]};
+    return __builtin_bit_cast(V8, v);
+  }
+};
+
+
+
 template <typename T, int R, int BK, bool KMAJOR, int NW>
 struct DmaPanel {
   static constexpr int CPR = KMAJOR ? BK / 8 : R / 8;
@@ -295,8 +321,8 @@ struct DmaPanel {
   static_assert(KMAJOR ? (CPR == 4 || CPR == 8) : (CPR >= 16), "unsupported panel shape");
 
   static __device__ __forceinline__ int swz(int lrow, int c) {
-    if (KMAJOR) return c ^ ((lrow / (16 / CPR)) % CPR);
-    return c ^ ((lrow & 3) << 2);
+    if constexpr (KMAJOR) return c ^ ((lrow / (16 / CPR)) % CPR);
+    else return c ^ ((lrow & 3) << 2);
   }
 
   // Global address of each of this lane's chunks for the step starting at kbeg.
@@ -322,6 +348,9 @@ struct DmaPanel {
     for (int j = 0; j < PER_WAVE; ++j)
       __builtin_amdgcn_global_load_lds((gptr_void*)ptrs[j], (lds_void*)(lds + (wave * PER_WAVE + j) * 1024), 16, 0, 0);
   }
+  static __device__ __forceinline__ void issue_one(const T* (&ptrs)[PER_WAVE], char* lds, int wave, int j) {
+    __builtin_amdgcn_global_load_lds((gptr_void*)ptrs[j], (lds_void*)(lds + (wave * PER_WAVE + j) * 1024), 16, 0, 0);
+  }
   static __device__ __forceinline__ void advance(const T* (&ptrs)[PER_WAVE], int64_t ld) {
 #pragma unroll
     for (int j = 0; j < PER_WAVE; ++j) ptrs[j] += KMAJOR ? (int64_t)BK : (int64_t)BK * ld;
@@ -329,14 +358,31 @@ struct DmaPanel {
   static __device__ __forceinline__ typename Vec<T>::v8 frag(const char* lds, int rb, int ks, int lane) {
     return Panel<T, R, BK, KMAJOR, 64, true>::frag(lds, rb, ks, lane);
   }
+  static constexpr int READS_PER_FRAG = KMAJOR ? 1 : 2;
+  // Same operand as frag(), read with volatile asm from the panel at LDS byte address `base`.
+  static __device__ __forceinline__ void frag_issue(FragRegs<KMAJOR>& f, uint32_t base, int rb, int ks, int lane) {
+    if constexpr (KMAJOR) {
+      const int row = rb + (lane & 31);
+      const int c = ks * 2 + (lane >> 5);
+      const uint32_t a = base + (row * CPR + swz(row, c)) * 16;
+      asm volatile("ds_read_b128 %0, %1" : "=v"(f.q) : "v"(a));
+    } else {
+      const int i = lane & 15;
+      const int col = rb + 16 * ((lane >> 4) & 1) + (i & 3) * 4;
+      const int kk0 = ks * 16 + 8 * (lane >> 5) + (i >> 2);
+      const int kk1 = kk0 + 4;
+      const uint32_t a0 = base + (kk0 * CPR + swz(kk0, col >> 3)) * 16 + (col & 7) * 2;
+      const uint32_t a1 = base + (kk1 * CPR + swz(kk1, col >> 3)) * 16 + (col & 7) * 2;
+      asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(f.lo) : "v"(a0));
+      asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(f.hi) : "v"(a1));
+    }
+  }
 };
 
 // s_waitcnt vmcnt(n) with the other counters unconstrained (gfx9 encoding).
 template <int N> __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
-
-
 // Epilogue of the direct-to-LDS kernel.  Each wave rounds its accumulators (after
 // bias / ReLU), parks one 32-row block at a time in a private LDS region and
 // reads it back row-contiguously, so every global store instruction writes whole
@@ -428,6 +474,7 @@ __global__ __launch_bounds__(WM* WN * 64, WPE) void gemm_dma_kernel(GemmParams p
   const int kend = min(p.K, kbeg + p.k_per_split);
   const int nk = (kend - kbeg) / BK;
 
+  if (p.flags & 16) return;
   const T* pa[PA::PER_WAVE];
   const T* pb[PB::PER_WAVE];
   PA::init(pa, (const T*)p.A, p.lda, m0, p.M, kbeg, wave, lane);
@@ -452,6 +499,7 @@ __global__ __launch_bounds__(WM* WN * 64, WPE) void gemm_dma_kernel(GemmParams p
     }
   }
 
+  if (p.flags & 32) return;
   int stage = 0;        // stage holding step kt
   int fill = D % STAGES;  // stage that step kt + D goes to
   for (int kt = 0; kt < nk; ++kt) {
@@ -466,47 +514,69 @@ __global__ __launch_bounds__(WM* WN * 64, WPE) void gemm_dma_kernel(GemmParams p
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    if (kt + D < nk && !(p.flags & 2)) {
-      PA::issue(pa, smem + fill * STAGE, wave);
-      PB::issue(pb, smem + fill * STAGE + PA::BYTES, wave);
-      PA::advance(pa, p.lda);
-      PB::advance(pb, p.ldb);
-    }
+    const bool prefetch = kt + D < nk && !(p.flags & 2);
+    char* fa_dst = smem + fill * STAGE;
+    char* fb_dst = fa_dst + PA::BYTES;
+    // this wave's loads of step kt+D are spread over the contraction steps below, so the
+    // memory pipeline sees a steady stream instead of a burst behind every barrier
+    auto issue_slice = [&](int ks) {
+      constexpr int KSTEPS_ = BK / 16;
+#pragma unroll
+      for (int q = 0; q < LPS; ++q) {
+        if (q * KSTEPS_ / LPS == ks) {
+          if (q < PA::PER_WAVE) PA::issue_one(pa, fa_dst, wave, q);
+          else PB::issue_one(pb, fb_dst, wave, q - PA::PER_WAVE);
+        }
+      }
+    };
     const char* sa = smem + stage * STAGE;
     const char* sb = sa + PA::BYTES;
-    if (p.flags & 4) continue;
-    // operands of contraction step ks+1 are read from LDS while the MFMAs of step ks run
-    v8 fa[2][TM], fb[2][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i) fa[0][i] = PA::frag(sa, wm * WTM + i * 32, 0, lane);
-#pragma unroll
-    for (int j = 0; j < TN; ++j) fb[0][j] = PB::frag(sb, wn * WTN + j * 32, 0, lane);
-#pragma unroll
-    for (int ks = 0; ks < BK / 16; ++ks) {
-      if (ks + 1 < BK / 16) {
-#pragma unroll
-        for (int i = 0; i < TM; ++i) fa[(ks + 1) & 1][i] = PA::frag(sa, wm * WTM + i * 32, ks + 1, lane);
-#pragma unroll
-        for (int j = 0; j < TN; ++j) fb[(ks + 1) & 1][j] = PB::frag(sb, wn * WTN + j * 32, ks + 1, lane);
+    if (p.flags & 4) {
+      if (prefetch) {
+        PA::issue(pa, fa_dst, wave);
+        PB::issue(pb, fb_dst, wave);
+        PA::advance(pa, p.lda);
+        PB::advance(pb, p.ldb);
       }
+      stage = stage + 1 == STAGES ? 0 : stage + 1;
+      fill = fill + 1 == STAGES ? 0 : fill + 1;
+      continue;
+    }
+    // Operands of contraction step ks+1 are requested from LDS before the MFMAs of
+    // step ks are issued, so their latency hides behind 8-16 MFMAs of this wave.
+    constexpr int KSTEPS = BK / 16;
+    constexpr int NREAD = TM * PA::READS_PER_FRAG + TN * PB::READS_PER_FRAG;
+    static_assert(NREAD <= 15, "lgkmcnt range");
+    const uint32_t sa_addr = lds_address(sa), sb_addr = lds_address(sb);
+    FragRegs<A_KMAJOR> fa[2][TM];
+    FragRegs<B_KMAJOR> fb[2][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) PA::frag_issue(fa[0][i], sa_addr, wm * WTM + i * 32, 0, lane);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) PB::frag_issue(fb[0][j], sb_addr, wn * WTN + j * 32, 0, lane);
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      if (ks + 1 < KSTEPS) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) PA::frag_issue(fa[(ks + 1) & 1][i], sa_addr, wm * WTM + i * 32, ks + 1, lane);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) PB::frag_issue(fb[(ks + 1) & 1][j], sb_addr, wn * WTN + j * 32, ks + 1, lane);
+        wait_lgkmcnt<NREAD>();  // step ks has landed; step ks+1 may still be in flight
+      } else {
+        wait_lgkmcnt<0>();
+      }
+      if (prefetch) issue_slice(ks);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j) acc[i][j] = mfma32(fb[ks & 1][j], fa[ks & 1][i], acc[i][j]);
-      // issue order within the step: the LDS reads of step ks+1 are spread between
-      // the MFMAs of step ks instead of being bunched in front of them
-      if (ks + 1 < BK / 16) {
-        constexpr int NREAD = TM * (A_KMAJOR ? 1 : 2) + TN * (B_KMAJOR ? 1 : 2);
-        constexpr int NMFMA = TM * TN;
-        constexpr int PER = NREAD >= NMFMA ? (NREAD + NMFMA - 1) / NMFMA : 1;  // reads after each MFMA
-        constexpr int SLOTS = (NREAD + PER - 1) / PER;
-#pragma unroll
-        for (int q = 0; q < SLOTS; ++q) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, PER, 0);
-        }
-        if (NMFMA > SLOTS) __builtin_amdgcn_sched_group_barrier(0x008, NMFMA - SLOTS, 0);
-      }
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = mfma32(fb[ks & 1][j].template get<v8>(), fa[ks & 1][i].template get<v8>(), acc[i][j]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (prefetch) {
+      PA::advance(pa, p.lda);
+      PB::advance(pb, p.ldb);
     }
     stage = stage + 1 == STAGES ? 0 : stage + 1;
     fill = fill + 1 == STAGES ? 0 : fill + 1;
@@ -584,6 +654,8 @@ static const TileCfg kCfgs[] = {
     {256, 128, 32, 4, 3},  // 9: 72 KB LDS, two workgroups per CU, wave tile 128x64
     {128, 256, 32, 4, 3},  // 10: as 9, wave tile 64x128
     {128, 128, 64, 4, 3},  // 11
+    {256, 128, 64, 8, 2},  // 12: 96 KB LDS, eight waves (4x2), wave tile 64x64
+    {128, 256, 64, 8, 2},  // 13: as 12 transposed (2x4 waves)
 };
 constexpr int kNumCfgs = (int)(sizeof(kCfgs) / sizeof(kCfgs[0]));
 
@@ -686,6 +758,8 @@ static int launch_cfg(hipStream_t st, const GemmPlan& pl, const GemmParams& p) {
       case 9: return launch_dma<T, 256, 128, 32, 2, 2, 3, 2, AK, BKM>(st, p);
       case 10: return launch_dma<T, 128, 256, 32, 2, 2, 3, 2, AK, BKM>(st, p);
       case 11: return launch_dma<T, 128, 128, 64, 2, 2, 3, 1, AK, BKM>(st, p);
+      case 12: return launch_dma<T, 256, 128, 64, 4, 2, 2, 2, AK, BKM>(st, p);
+      case 13: return launch_dma<T, 128, 256, 64, 2, 4, 2, 2, AK, BKM>(st, p);
     }
   }
   // fallbacks with the same tile shape where one exists
