@@ -86,9 +86,8 @@ int64_t tf_gemm_workspace_bytes(int layout_a, int layout_b, int64_t M, int64_t N
  * (-1 = automatic) and contraction split `splits` (0 = automatic) for all
  * later tf_gemm / tf_gemm_workspace_bytes calls of this process. */
 int tf_gemm_tune(int cfg, int splits);
-/* Diagnostic: bit 0 disables the XCD-aware workgroup remap, bit 1 skips the
- * in-loop operand loads, bit 2 skips the MFMA work (bits 1-2 give WRONG results;
- * they exist to time the pipeline's parts in isolation). */
+/* Diagnostic: bit 0 disables the XCD-aware workgroup remap; bit 3 skips the
+ * result write-out (WRONG results: it exists to time the main loop alone). */
 int tf_gemm_debug_flags(int flags);
 
 /* Causal flash attention forward.  q,k,v,o: logical (B, nh, S, hd) with the

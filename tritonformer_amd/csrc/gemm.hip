@@ -440,19 +440,21 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x16 (&
   }
 }
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES, int WPE, bool A_KMAJOR, bool B_KMAJOR>
+template <typename T, int BM, int BN, int BK, int WM, int WN, int WPE, bool A_KMAJOR, bool B_KMAJOR>
 __global__ __launch_bounds__(WM* WN * 64, WPE) void gemm_dma_kernel(GemmParams p) {
   constexpr int NW = WM * WN;
   constexpr int WTM = BM / WM, WTN = BN / WN;
   constexpr int TM = WTM / 32, TN = WTN / 32;
   constexpr int GROUP_M = 8;
-  constexpr int D = STAGES - 1;  // prefetch distance
+  constexpr int KSTEPS = BK / 16;
   typedef DmaPanel<T, BM, BK, A_KMAJOR, NW> PA;
   typedef DmaPanel<T, BN, BK, B_KMAJOR, NW> PB;
   typedef typename Vec<T>::v8 v8;
-  constexpr int STAGE = PA::BYTES + PB::BYTES;
+  constexpr int STAGE = PA::BYTES + PB::BYTES;      // two stages, ping-pong
   constexpr int LPS = PA::PER_WAVE + PB::PER_WAVE;  // loads per wave per stage
-  static_assert(LPS * D < 64, "vmcnt range");
+  constexpr int NREAD = TM * PA::READS_PER_FRAG + TN * PB::READS_PER_FRAG;  // LDS reads per contraction step
+  static_assert(NREAD <= 15, "lgkmcnt range");
+  static_assert(KSTEPS % 2 == 0, "operand register ping-pong needs an even number of contraction steps");
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   const int lane = threadIdx.x & 63;
@@ -474,7 +476,6 @@ __global__ __launch_bounds__(WM* WN * 64, WPE) void gemm_dma_kernel(GemmParams p
   const int kend = min(p.K, kbeg + p.k_per_split);
   const int nk = (kend - kbeg) / BK;
 
-  if (p.flags & 16) return;
   const T* pa[PA::PER_WAVE];
   const T* pb[PB::PER_WAVE];
   PA::init(pa, (const T*)p.A, p.lda, m0, p.M, kbeg, wave, lane);
@@ -488,84 +489,71 @@ __global__ __launch_bounds__(WM* WN * 64, WPE) void gemm_dma_kernel(GemmParams p
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  // prologue: D steps in flight
-#pragma unroll
-  for (int s = 0; s < D; ++s) {
-    if (s < nk) {
-      PA::issue(pa, smem + s * STAGE, wave);
-      PB::issue(pb, smem + s * STAGE + PA::BYTES, wave);
-      PA::advance(pa, p.lda);
-      PB::advance(pb, p.ldb);
-    }
-  }
-
-  if (p.flags & 32) return;
-  int stage = 0;        // stage holding step kt
-  int fill = D % STAGES;  // stage that step kt + D goes to
-  for (int kt = 0; kt < nk; ++kt) {
-    // this wave's loads of step kt have landed once at most the later steps' loads are outstanding
-    const int later = min(D - 1, nk - 1 - kt);
-    if (later >= 2) wait_vmcnt<LPS * 2>();
-    else if (later == 1) wait_vmcnt<LPS * (D >= 2 ? 1 : 0)>();
-    else wait_vmcnt<0>();
-    // Bare s_barrier: __syncthreads() would add a fence that drains every outstanding
-    // direct-to-LDS load.  The waits that matter are explicit: this wave's loads of
-    // step kt (above) and its LDS reads of step kt-1 (consumed by the MFMAs already).
+  // Bare s_barrier everywhere in the pipeline: __syncthreads() adds a fence that would
+  // drain every outstanding direct-to-LDS load.  The waits that matter are explicit.
+  auto barrier = [&]() {
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    const bool prefetch = kt + D < nk && !(p.flags & 2);
-    char* fa_dst = smem + fill * STAGE;
-    char* fb_dst = fa_dst + PA::BYTES;
-    // this wave's loads of step kt+D are spread over the contraction steps below, so the
-    // memory pipeline sees a steady stream instead of a burst behind every barrier
-    auto issue_slice = [&](int ks) {
-      constexpr int KSTEPS_ = BK / 16;
+  };
+  // slice sl (of KSTEPS) of this wave's loads of one contraction step, into stage `dst`
+  auto issue_slice = [&](char* dst, int sl) {
 #pragma unroll
-      for (int q = 0; q < LPS; ++q) {
-        if (q * KSTEPS_ / LPS == ks) {
-          if (q < PA::PER_WAVE) PA::issue_one(pa, fa_dst, wave, q);
-          else PB::issue_one(pb, fb_dst, wave, q - PA::PER_WAVE);
-        }
+    for (int q = 0; q < LPS; ++q) {
+      if (q * KSTEPS / LPS == sl) {
+        if (q < PA::PER_WAVE) PA::issue_one(pa, dst, wave, q);
+        else PB::issue_one(pb, dst + PA::BYTES, wave, q - PA::PER_WAVE);
       }
-    };
-    const char* sa = smem + stage * STAGE;
-    const char* sb = sa + PA::BYTES;
-    if (p.flags & 4) {
-      if (prefetch) {
-        PA::issue(pa, fa_dst, wave);
-        PB::issue(pb, fb_dst, wave);
-        PA::advance(pa, p.lda);
-        PB::advance(pb, p.ldb);
-      }
-      stage = stage + 1 == STAGES ? 0 : stage + 1;
-      fill = fill + 1 == STAGES ? 0 : fill + 1;
-      continue;
     }
-    // Operands of contraction step ks+1 are requested from LDS before the MFMAs of
-    // step ks are issued, so their latency hides behind 8-16 MFMAs of this wave.
-    constexpr int KSTEPS = BK / 16;
-    constexpr int NREAD = TM * PA::READS_PER_FRAG + TN * PB::READS_PER_FRAG;
-    static_assert(NREAD <= 15, "lgkmcnt range");
-    const uint32_t sa_addr = lds_address(sa), sb_addr = lds_address(sb);
-    FragRegs<A_KMAJOR> fa[2][TM];
-    FragRegs<B_KMAJOR> fb[2][TN];
+  };
+  FragRegs<A_KMAJOR> fa[2][TM];
+  FragRegs<B_KMAJOR> fb[2][TN];
+  auto read_operands = [&](const char* stage, int ks, int buf) {
+    const uint32_t sa_addr = lds_address(stage), sb_addr = sa_addr + PA::BYTES;
 #pragma unroll
-    for (int i = 0; i < TM; ++i) PA::frag_issue(fa[0][i], sa_addr, wm * WTM + i * 32, 0, lane);
+    for (int i = 0; i < TM; ++i) PA::frag_issue(fa[buf][i], sa_addr, wm * WTM + i * 32, ks, lane);
 #pragma unroll
-    for (int j = 0; j < TN; ++j) PB::frag_issue(fb[0][j], sb_addr, wn * WTN + j * 32, 0, lane);
+    for (int j = 0; j < TN; ++j) PB::frag_issue(fb[buf][j], sb_addr, wn * WTN + j * 32, ks, lane);
+  };
+
+  // ---- prologue: step 0 into stage 0, then its first operands and the head of step 1
+  if (nk > 0) {
+    PA::issue(pa, smem, wave);
+    PB::issue(pb, smem + PA::BYTES, wave);
+    PA::advance(pa, p.lda);
+    PB::advance(pb, p.ldb);
+    wait_vmcnt<0>();
+    barrier();
+    read_operands(smem, 0, 0);
+    if (nk > 1) issue_slice(smem + STAGE, 0);
+  }
+
+  // ---- main loop.  Per step of BK: the operands of contraction step ks+1 are requested
+  // from LDS before the MFMAs of step ks are issued; the loads of the next BK step
+  // trickle in slice by slice; and the hand-over to the next stage (wait for the loads,
+  // barrier, first operand reads of the next stage, head of the step after) happens
+  // BEFORE the last group of MFMAs, so no MFMA ever waits on a freshly issued LDS read.
+  for (int kt = 0; kt < nk; ++kt) {
+    char* cur = smem + (kt & 1) * STAGE;
+    char* nxt = smem + ((kt + 1) & 1) * STAGE;
+    const bool more = kt + 1 < nk;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
       if (ks + 1 < KSTEPS) {
-#pragma unroll
-        for (int i = 0; i < TM; ++i) PA::frag_issue(fa[(ks + 1) & 1][i], sa_addr, wm * WTM + i * 32, ks + 1, lane);
-#pragma unroll
-        for (int j = 0; j < TN; ++j) PB::frag_issue(fb[(ks + 1) & 1][j], sb_addr, wn * WTN + j * 32, ks + 1, lane);
+        read_operands(cur, ks + 1, (ks + 1) & 1);
         wait_lgkmcnt<NREAD>();  // step ks has landed; step ks+1 may still be in flight
+        if (more) issue_slice(nxt, ks + 1);
       } else {
-        wait_lgkmcnt<0>();
+        wait_lgkmcnt<0>();      // every LDS read of this stage is complete
+        if (more) {
+          PA::advance(pa, p.lda);
+          PB::advance(pb, p.ldb);
+          wait_vmcnt<0>();      // this wave's loads of the next stage have landed
+          barrier();            // ... and everyone's; everyone is done reading `cur`
+          read_operands(nxt, 0, 0);
+          if (kt + 2 < nk) issue_slice(cur, 0);
+        }
       }
-      if (prefetch) issue_slice(ks);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < TM; ++i)
@@ -574,19 +562,13 @@ __global__ __launch_bounds__(WM* WN * 64, WPE) void gemm_dma_kernel(GemmParams p
           acc[i][j] = mfma32(fb[ks & 1][j].template get<v8>(), fa[ks & 1][i].template get<v8>(), acc[i][j]);
       __builtin_amdgcn_sched_barrier(0);
     }
-    if (prefetch) {
-      PA::advance(pa, p.lda);
-      PB::advance(pb, p.ldb);
-    }
-    stage = stage + 1 == STAGES ? 0 : stage + 1;
-    fill = fill + 1 == STAGES ? 0 : fill + 1;
   }
 
   if (p.flags & 8) return;
   if (p.splits > 1) {
     gemm_epilogue<T, TM, TN, WTM, WTN, true>(p, acc, m0, n0, wm, wn, lane, split);
   } else {
-    static_assert(NW * 32 * (WTN * 4 + 16) <= STAGES * STAGE, "epilogue staging must fit in the pipeline LDS");
+    static_assert(NW * 32 * (WTN * 4 + 16) <= 2 * STAGE, "epilogue staging must fit in the pipeline LDS");
     __syncthreads();  // all waves are done reading the last pipeline stage
     if (p.out_f32) gemm_epilogue_lds<T, float, TM, TN, WTM, WTN>(p, acc, smem, m0, n0, wm, wn, wave, lane);
     else gemm_epilogue_lds<T, T, TM, TN, WTM, WTN>(p, acc, smem, m0, n0, wm, wn, wave, lane);
@@ -639,23 +621,15 @@ struct GemmPlan {
   int tiles_m, tiles_n, splits, k_per_split;
 };
 
-struct TileCfg { int bm, bn, bk, waves, stages; };  // stages > 0: direct-to-LDS kernel
+struct TileCfg { int bm, bn, bk, waves, dma; };  // dma: direct-to-LDS kernel
 // index = cfg id used by launch_cfg below
 static const TileCfg kCfgs[] = {
-    {256, 256, 64, 8, 0},  // 0: register-staged, wave tile 128x64
-    {128, 128, 64, 4, 0},  // 1: register-staged, wave tile 64x64
-    {256, 256, 32, 8, 4},  // 2: direct-to-LDS, 4 stages, wave tile 128x64
-    {256, 128, 32, 4, 4},  // 3: direct-to-LDS, 4 stages, wave tile 128x64
-    {256, 256, 32, 8, 3},  // 4
-    {128, 128, 32, 4, 4},  // 5: wave tile 64x64
-    {256, 128, 64, 4, 3},  // 6
-    {256, 256, 64, 8, 2},  // 7
-    {128, 128, 64, 4, 2},  // 8: 64 KB LDS, two workgroups per CU
-    {256, 128, 32, 4, 3},  // 9: 72 KB LDS, two workgroups per CU, wave tile 128x64
-    {128, 256, 32, 4, 3},  // 10: as 9, wave tile 64x128
-    {128, 128, 64, 4, 3},  // 11
-    {256, 128, 64, 8, 2},  // 12: 96 KB LDS, eight waves (4x2), wave tile 64x64
-    {128, 256, 64, 8, 2},  // 13: as 12 transposed (2x4 waves)
+    {256, 256, 64, 8, 0},  // 0: register-staged, wave tile 128x64, any shape / alignment
+    {128, 128, 64, 4, 0},  // 1: register-staged, wave tile 64x64, any shape / alignment
+    {256, 256, 64, 8, 1},  // 2: direct-to-LDS, 128 KB LDS, one workgroup per CU, wave tile 128x64
+    {128, 128, 64, 4, 1},  // 3: direct-to-LDS, 64 KB LDS, two workgroups per CU, wave tile 64x64
+    {256, 128, 64, 8, 1},  // 4: direct-to-LDS, 96 KB LDS, waves 4x2, wave tile 64x64
+    {128, 256, 64, 8, 1},  // 5: direct-to-LDS, 96 KB LDS, waves 2x4, wave tile 64x64
 };
 constexpr int kNumCfgs = (int)(sizeof(kCfgs) / sizeof(kCfgs[0]));
 
@@ -672,14 +646,16 @@ static GemmPlan make_plan(int64_t M, int64_t N, int64_t K, bool vec) {
   const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
   // Measured on MI355X (gfx950): 256x256 tiles win once they alone give every CU
   // work, and for long contractions over a mid-sized output (weight gradients of
-  // the MLP) when combined with a contraction split; everything else runs
-  // 128x128 tiles with two workgroups resident per CU.
+  // the MLP) when combined with a contraction split; smaller outputs run 256x128
+  // tiles (one workgroup of eight waves per CU), very long contractions over a small
+  // output 128x128 tiles with two workgroups resident per CU.
   const bool dma = vec && K % 64 == 0;
   const bool long_k_mid = big_tiles >= 48 && big_tiles < 128 && K >= 4096 && K >= 2 * (M > N ? M : N);
-  if (big_tiles >= 200 || long_k_mid) pl.cfg = dma ? 7 : 0;
-  else pl.cfg = dma ? 8 : 1;
+  if (big_tiles >= 200 || long_k_mid) pl.cfg = dma ? 2 : 0;
+  else if (dma) pl.cfg = K >= 16384 ? 3 : 4;
+  else pl.cfg = 1;
   if (g_force_cfg >= 0 && g_force_cfg < kNumCfgs) pl.cfg = g_force_cfg;
-  if (kCfgs[pl.cfg].stages > 0 && !(vec && K % kCfgs[pl.cfg].bk == 0))
+  if (kCfgs[pl.cfg].dma && !(vec && K % kCfgs[pl.cfg].bk == 0))
     pl.cfg = kCfgs[pl.cfg].bm * kCfgs[pl.cfg].bn >= 256 * 256 ? 0 : 1;  // register-staged twin
   pl.bm = kCfgs[pl.cfg].bm;
   pl.bn = kCfgs[pl.cfg].bn;
@@ -727,11 +703,11 @@ static int launch_one(hipStream_t st, const GemmParams& p) {
   return TF_OK;
 }
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES, int WPE, bool AK, bool BKM>
+template <typename T, int BM, int BN, int BK, int WM, int WN, int WPE, bool AK, bool BKM>
 static int launch_dma(hipStream_t st, const GemmParams& p) {
-  constexpr int lds = STAGES * (BM + BN) * BK * 2;
+  constexpr int lds = 2 * (BM + BN) * BK * 2;
   static_assert(lds <= 160 * 1024, "LDS budget");
-  auto kernel = gemm_dma_kernel<T, BM, BN, BK, WM, WN, STAGES, WPE, AK, BKM>;
+  auto kernel = gemm_dma_kernel<T, BM, BN, BK, WM, WN, WPE, AK, BKM>;
   static bool once = (allow_big_lds(kernel, lds), true);
   (void)once;
   const unsigned grid = (unsigned)(p.tiles_m * p.tiles_n * p.splits);
@@ -745,26 +721,16 @@ static int launch_dma(hipStream_t st, const GemmParams& p) {
 // contraction extent that is a multiple of its BK.
 template <typename T, bool AK, bool BKM, bool VEC>
 static int launch_cfg(hipStream_t st, const GemmPlan& pl, const GemmParams& p) {
-  const bool dma_ok = VEC && p.K % pl.bk == 0;
-  if (kCfgs[pl.cfg].stages > 0 && dma_ok) {
+  if (kCfgs[pl.cfg].dma && VEC && p.K % pl.bk == 0) {
     switch (pl.cfg) {
-      case 2: return launch_dma<T, 256, 256, 32, 2, 4, 4, 2, AK, BKM>(st, p);
-      case 3: return launch_dma<T, 256, 128, 32, 2, 2, 4, 1, AK, BKM>(st, p);
-      case 4: return launch_dma<T, 256, 256, 32, 2, 4, 3, 2, AK, BKM>(st, p);
-      case 5: return launch_dma<T, 128, 128, 32, 2, 2, 4, 2, AK, BKM>(st, p);
-      case 6: return launch_dma<T, 256, 128, 64, 2, 2, 3, 1, AK, BKM>(st, p);
-      case 7: return launch_dma<T, 256, 256, 64, 2, 4, 2, 2, AK, BKM>(st, p);
-      case 8: return launch_dma<T, 128, 128, 64, 2, 2, 2, 2, AK, BKM>(st, p);
-      case 9: return launch_dma<T, 256, 128, 32, 2, 2, 3, 2, AK, BKM>(st, p);
-      case 10: return launch_dma<T, 128, 256, 32, 2, 2, 3, 2, AK, BKM>(st, p);
-      case 11: return launch_dma<T, 128, 128, 64, 2, 2, 3, 1, AK, BKM>(st, p);
-      case 12: return launch_dma<T, 256, 128, 64, 4, 2, 2, 2, AK, BKM>(st, p);
-      case 13: return launch_dma<T, 128, 256, 64, 2, 4, 2, 2, AK, BKM>(st, p);
+      case 2: return launch_dma<T, 256, 256, 64, 2, 4, 2, AK, BKM>(st, p);
+      case 3: return launch_dma<T, 128, 128, 64, 2, 2, 2, AK, BKM>(st, p);
+      case 4: return launch_dma<T, 256, 128, 64, 4, 2, 2, AK, BKM>(st, p);
+      case 5: return launch_dma<T, 128, 256, 64, 2, 4, 2, AK, BKM>(st, p);
     }
   }
-  // fallbacks with the same tile shape where one exists
-  if (pl.bm == 256 && pl.bn == 256 && pl.bk == 64) return launch_one<T, 256, 256, 64, 2, 4, AK, BKM, VEC>(st, p);
-  if (pl.bm == 128 && pl.bn == 128 && pl.bk == 64) return launch_one<T, 128, 128, 64, 2, 2, AK, BKM, VEC>(st, p);
+  if (pl.bm == 256 && pl.bn == 256) return launch_one<T, 256, 256, 64, 2, 4, AK, BKM, VEC>(st, p);
+  if (pl.bm == 128 && pl.bn == 128) return launch_one<T, 128, 128, 64, 2, 2, AK, BKM, VEC>(st, p);
   return TF_EINVAL;
 }
 
@@ -810,7 +776,7 @@ extern "C" int tf_gemm_tune(int cfg, int splits) {
   return TF_OK;
 }
 
-// Diagnostic: bit 0 skips the XCD remap, bit 1 skips the in-loop loads, bit 2 the MFMA work.
+// Diagnostic: bit 0 skips the XCD remap, bit 3 skips the epilogue (timing only, wrong results).
 extern "C" int tf_gemm_debug_flags(int flags) {
   g_flags = flags;
   return TF_OK;
