@@ -23,6 +23,10 @@
 #include <cstdlib>
 #include "rowops.h"
 
+#ifndef TF_GEMM_NSLICE
+#define TF_GEMM_NSLICE 2  // the loads of the next step go out in this many slices, early in the step
+#endif
+
 namespace tfa {
 
 struct GemmParams {
@@ -496,11 +500,13 @@ __global__ __launch_bounds__(WM* WN * 64, WPE) void gemm_dma_kernel(GemmParams p
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
   };
-  // slice sl (of KSTEPS) of this wave's loads of one contraction step, into stage `dst`
+  // slice sl (of NSLICE) of this wave's loads of one contraction step, into stage `dst`;
+  // slices >= NSLICE are empty
+  constexpr int NSLICE = TF_GEMM_NSLICE < KSTEPS ? TF_GEMM_NSLICE : KSTEPS;
   auto issue_slice = [&](char* dst, int sl) {
 #pragma unroll
     for (int q = 0; q < LPS; ++q) {
-      if (q * KSTEPS / LPS == sl) {
+      if (q * NSLICE / LPS == sl) {
         if (q < PA::PER_WAVE) PA::issue_one(pa, dst, wave, q);
         else PB::issue_one(pb, dst + PA::BYTES, wave, q - PA::PER_WAVE);
       }
