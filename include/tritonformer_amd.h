@@ -151,19 +151,25 @@ int tf_softmax_bwd(void* stream, int dtype, int64_t rows, int64_t cols,
 /* Per-row loss[r] = logsumexp(logits[r,:]) - logits[r, labels[r]] with an
  * online max/sum single pass; also stores lse[r] (natural log, fp32).
  * labels: int64, each in [0, V).  loss has `dtype`.
+ * Row r starts at element (r / inner_rows) * outer_stride + (r % inner_rows) * ld;
+ * inner_rows <= 0 means a plain matrix (row r at r * ld).  With inner_rows = S-1,
+ * ld = V, outer_stride = S*V the rows are those of a (B, S, V) tensor without the
+ * last position of each sequence: the shifted logits of transformer.py:333 read
+ * in place, without the .contiguous() copy.
  * Replaces cross_entropy_fwd (kernels/crossentropy.py:47-75). */
 int tf_cross_entropy_fwd(void* stream, int dtype, int64_t rows, int64_t V,
-                         const void* logits, int64_t ld, const int64_t* labels,
-                         void* loss, float* lse);
+                         const void* logits, int64_t ld, int64_t inner_rows, int64_t outer_stride,
+                         const int64_t* labels, void* loss, float* lse);
 
-/* dlogits[r,v] = (exp(logits[r,v] - lse[r]) - [v == labels[r]]) * gout[r].
+/* dlogits[r,v] = (exp(logits[r,v] - lse[r]) - [v == labels[r]]) * gout[r], rows of
+ * dlogits addressed like those of logits with (ldd, inner_rows, outer_stride_d).
  * Replaces cross_entropy_bwd (kernels/crossentropy.py:110-127) and the
  * broadcast multiply in tritonformer/crossentropy.py:24.  gout has `dtype`;
  * gout_stride 0 broadcasts one value. */
 int tf_cross_entropy_bwd(void* stream, int dtype, int64_t rows, int64_t V,
-                         const void* logits, int64_t ld, const int64_t* labels,
-                         const float* lse, const void* gout, int64_t gout_stride,
-                         void* dlogits, int64_t ldd);
+                         const void* logits, int64_t ld, int64_t inner_rows, int64_t outer_stride,
+                         const int64_t* labels, const float* lse, const void* gout, int64_t gout_stride,
+                         void* dlogits, int64_t ldd, int64_t outer_stride_d);
 
 /* out[c] = sum_r x[r, c] with fp32 accumulation (bias gradient).
  * Replaces unbroadcast_leading (kernels/reductions.py:97-122, two-stage with

@@ -93,13 +93,14 @@ def test_row_kernels_reject_bad_arguments():
                                 None, 0) == -5
     assert lib.tf_layernorm_bwd_partial_bytes(8192, 1024) == 512 * 2 * 1024 * 4
     assert lib.tf_softmax_fwd(None, 0, 4, 0, FAKE, 64, FAKE, 64) == -1
-    assert lib.tf_cross_entropy_fwd(None, 2, 4, 64, FAKE, 64, FAKE, FAKE, FAKE) == -2
-    assert lib.tf_cross_entropy_bwd(None, 0, 4, 64, FAKE, 32, FAKE, FAKE, FAKE, 1, FAKE, 64) == -1
+    assert lib.tf_cross_entropy_fwd(None, 2, 4, 64, FAKE, 64, 0, 0, FAKE, FAKE, FAKE) == -2
+    assert lib.tf_cross_entropy_bwd(None, 0, 4, 64, FAKE, 32, 0, 0, FAKE, FAKE, FAKE, 1, FAKE, 64, 0) == -1
+    assert lib.tf_cross_entropy_fwd(None, 0, 6, 64, FAKE, 64, 3, 100, FAKE, FAKE, FAKE) == -1   # groups overlap
     assert lib.tf_colsum(None, 0, 16, 64, FAKE, 64, FAKE, None, 0) == -5
     assert lib.tf_relu_mask(None, 0, 4, 64, None, 64, FAKE, 64, FAKE, 64) == -1
     # empty inputs are accepted and launch nothing
     assert lib.tf_softmax_fwd(None, 0, 0, 64, FAKE, 64, FAKE, 64) == 0
-    assert lib.tf_cross_entropy_fwd(None, 0, 0, 64, FAKE, 64, FAKE, FAKE, FAKE) == 0
+    assert lib.tf_cross_entropy_fwd(None, 0, 0, 64, FAKE, 64, 0, 0, FAKE, FAKE, FAKE) == 0
     assert lib.tf_relu_mask(None, 0, 0, 64, FAKE, 64, FAKE, 64, FAKE, 64) == 0
 
 

@@ -76,3 +76,25 @@ def test_argument_checks(dev):
         T.cross_entropy_loss.apply(torch.zeros(4, 8, device=dev, dtype=torch.float16), torch.zeros(4, device=dev, dtype=torch.int32))
     with pytest.raises(ValueError):
         T.cross_entropy_loss.apply(torch.zeros(4, 8, device=dev, dtype=torch.float16), torch.zeros(5, device=dev, dtype=torch.int64))
+
+
+@pytest.mark.parametrize("dims", [(2, 5, 904), (3, 64, 1000), (4, 256, 50304)])
+def test_shifted_cross_entropy_equals_copy_then_cross_entropy(dims, dev):
+    """The in-place shifted variant must give exactly what the reference's
+    shift-copy followed by the plain Function gives (transformer.py:333-341)."""
+    b, s, v = dims
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(b, s, v, generator=g).half().to(dev)
+    lab = torch.randint(0, v, (b, s), generator=g).to(dev)
+    xa = x.clone().requires_grad_(True)
+    xb = x.clone().requires_grad_(True)
+    fused = T.shifted_cross_entropy_loss.apply(xa, lab)
+    plain = T.cross_entropy_loss.apply(xb[:, :-1].contiguous().view(-1, v), lab[:, 1:].contiguous().view(-1))
+    assert fused.shape == (b * (s - 1),) and torch.equal(fused, plain)
+    gout = torch.randn(b * (s - 1), generator=g).half().to(dev)
+    fused.backward(gout)
+    plain.backward(gout)
+    assert torch.equal(xa.grad, xb.grad)
+    assert (xa.grad[:, -1] == 0).all()
+    ref = R.cross_entropy(x[:, :-1].reshape(-1, v).cpu(), lab[:, 1:].reshape(-1).cpu())
+    assert_close(fused, ref, name="shifted loss")

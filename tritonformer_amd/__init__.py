@@ -6,6 +6,7 @@ exports, backed by hand-written HIP kernels behind a C ABI."""
 from .attention import BiasedCausalAttention as fast_causal_attention_with_bias
 from .attention import CausalAttention as fast_causal_attention
 from .crossentropy import CrossEntropyLoss as cross_entropy_loss
+from .crossentropy import ShiftedCrossEntropyLoss as shifted_cross_entropy_loss
 from .layernorm import LayerNorm as layer_norm
 from .linear import LinearBias as linear_bias
 from .linear import LinearBiasReLU as linear_fused_bias_relu

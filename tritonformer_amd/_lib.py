@@ -34,8 +34,8 @@ SIGNATURES = {
     "tf_layernorm_bwd_partial_bytes": (_i64, [_i64, _i64]),
     "tf_softmax_fwd": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _vp, _i64]),
     "tf_softmax_bwd": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64]),
-    "tf_cross_entropy_fwd": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _vp, _vp, _vp]),
-    "tf_cross_entropy_bwd": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _vp, _i64]),
+    "tf_cross_entropy_fwd": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _i64, _i64, _vp, _vp, _vp]),
+    "tf_cross_entropy_bwd": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _i64, _vp, _i64, _i64]),
     "tf_colsum": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _vp, _vp, _i64]),
     "tf_colsum_partial_bytes": (_i64, [_i64, _i64]),
     "tf_relu_mask": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64]),

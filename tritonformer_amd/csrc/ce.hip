@@ -38,13 +38,22 @@ __device__ __forceinline__ MaxSum block_combine(MaxSum v, MaxSum* smem) {
   return r;
 }
 
+// Row r of the (rows, V) problem lives at (r / inner) * outer + (r % inner) * ld: with
+// inner = S-1, ld = V, outer = S*V these are the rows of a (B, S, V) tensor without the
+// last position of every sequence, i.e. the shifted logits read in place.
+struct RowMap {
+  int64_t ld, outer;
+  int inner;
+  __device__ __forceinline__ int64_t at(int64_t r) const { return (r / inner) * outer + (r % inner) * ld; }
+};
+
 template <typename T, bool VEC>
-__global__ __launch_bounds__(kCeThreads) void ce_fwd(int V, const T* __restrict__ logits, int64_t ld,
+__global__ __launch_bounds__(kCeThreads) void ce_fwd(int V, const T* __restrict__ logits, RowMap map,
                                                       const int64_t* __restrict__ labels, T* __restrict__ loss,
                                                       float* __restrict__ lse) {
   __shared__ MaxSum smem[kCeThreads / 64];
   const int64_t row = blockIdx.x;
-  const T* xr = logits + row * ld;
+  const T* xr = logits + map.at(row);
   MaxSum acc = {-INFINITY, 0.f};
   if (VEC) {
     const int nchunk = V >> 3;
@@ -79,13 +88,13 @@ __global__ __launch_bounds__(kCeThreads) void ce_fwd(int V, const T* __restrict_
 }
 
 template <typename T, bool VEC>
-__global__ __launch_bounds__(kCeThreads) void ce_bwd(int V, const T* __restrict__ logits, int64_t ld,
+__global__ __launch_bounds__(kCeThreads) void ce_bwd(int V, const T* __restrict__ logits, RowMap map,
                                                       const int64_t* __restrict__ labels,
                                                       const float* __restrict__ lse, const T* __restrict__ gout,
-                                                      int64_t gstride, T* __restrict__ dlogits, int64_t ldd) {
+                                                      int64_t gstride, T* __restrict__ dlogits, RowMap dmap) {
   const int64_t row = blockIdx.x;
-  const T* xr = logits + row * ld;
-  T* dr = dlogits + row * ldd;
+  const T* xr = logits + map.at(row);
+  T* dr = dlogits + dmap.at(row);
   const float l2 = lse[row] * kLog2e;
   const float g = (float)gout[row * gstride];
   const int lab = (int)labels[row];
@@ -114,28 +123,29 @@ __global__ __launch_bounds__(kCeThreads) void ce_bwd(int V, const T* __restrict_
 }
 
 template <typename T>
-static int ce_fwd_launch(hipStream_t st, int64_t rows, int64_t V, const void* logits, int64_t ld,
+static int ce_fwd_launch(hipStream_t st, int64_t rows, int64_t V, const void* logits, RowMap map,
                          const int64_t* labels, void* loss, float* lse) {
   const dim3 grid((unsigned)rows), block(kCeThreads);
-  if (row_vectorizable<T>(logits, V, ld))
-    ce_fwd<T, true><<<grid, block, 0, st>>>((int)V, (const T*)logits, ld, labels, (T*)loss, lse);
+  if (row_vectorizable<T>(logits, V, map.ld) && map.outer % 8 == 0)
+    ce_fwd<T, true><<<grid, block, 0, st>>>((int)V, (const T*)logits, map, labels, (T*)loss, lse);
   else
-    ce_fwd<T, false><<<grid, block, 0, st>>>((int)V, (const T*)logits, ld, labels, (T*)loss, lse);
+    ce_fwd<T, false><<<grid, block, 0, st>>>((int)V, (const T*)logits, map, labels, (T*)loss, lse);
   TF_CHECK_LAUNCH();
   return TF_OK;
 }
 
 template <typename T>
-static int ce_bwd_launch(hipStream_t st, int64_t rows, int64_t V, const void* logits, int64_t ld,
+static int ce_bwd_launch(hipStream_t st, int64_t rows, int64_t V, const void* logits, RowMap map,
                          const int64_t* labels, const float* lse, const void* gout, int64_t gstride,
-                         void* dlogits, int64_t ldd) {
+                         void* dlogits, RowMap dmap) {
   const dim3 grid((unsigned)rows), block(kCeThreads);
-  if (row_vectorizable<T>(logits, V, ld) && row_vectorizable<T>(dlogits, V, ldd))
-    ce_bwd<T, true><<<grid, block, 0, st>>>((int)V, (const T*)logits, ld, labels, lse, (const T*)gout, gstride,
-                                            (T*)dlogits, ldd);
+  if (row_vectorizable<T>(logits, V, map.ld) && row_vectorizable<T>(dlogits, V, dmap.ld) && map.outer % 8 == 0 &&
+      dmap.outer % 8 == 0)
+    ce_bwd<T, true><<<grid, block, 0, st>>>((int)V, (const T*)logits, map, labels, lse, (const T*)gout, gstride,
+                                            (T*)dlogits, dmap);
   else
-    ce_bwd<T, false><<<grid, block, 0, st>>>((int)V, (const T*)logits, ld, labels, lse, (const T*)gout, gstride,
-                                             (T*)dlogits, ldd);
+    ce_bwd<T, false><<<grid, block, 0, st>>>((int)V, (const T*)logits, map, labels, lse, (const T*)gout, gstride,
+                                             (T*)dlogits, dmap);
   TF_CHECK_LAUNCH();
   return TF_OK;
 }
@@ -144,28 +154,41 @@ static int ce_bwd_launch(hipStream_t st, int64_t rows, int64_t V, const void* lo
 
 using namespace tfa;
 
+static bool make_map(RowMap& m, int64_t rows, int64_t V, int64_t ld, int64_t inner, int64_t outer) {
+  if (inner <= 0) { inner = rows > 0 ? rows : 1; outer = 0; }
+  if (ld < V || inner > 0x7fffffff || outer < 0 || (inner < rows && outer < (inner - 1) * ld + V)) return false;
+  m.ld = ld; m.outer = outer; m.inner = (int)inner;
+  return true;
+}
+
 extern "C" int tf_cross_entropy_fwd(void* stream, int dtype, int64_t rows, int64_t V, const void* logits,
-                                    int64_t ld, const int64_t* labels, void* loss, float* lse) {
+                                    int64_t ld, int64_t inner_rows, int64_t outer_stride, const int64_t* labels,
+                                    void* loss, float* lse) {
   if (!logits || !labels || !loss || !lse) return TF_EINVAL;
-  if (rows < 0 || rows > 0x7fffffff || V <= 0 || V > (1 << 30) || ld < V) return TF_EINVAL;
+  if (rows < 0 || rows > 0x7fffffff || V <= 0 || V > (1 << 30)) return TF_EINVAL;
+  RowMap map;
+  if (!make_map(map, rows, V, ld, inner_rows, outer_stride)) return TF_EINVAL;
   if (rows == 0) return TF_OK;
   hipStream_t st = (hipStream_t)stream;
-  if (dtype == TF_F16) return ce_fwd_launch<f16>(st, rows, V, logits, ld, labels, loss, lse);
-  if (dtype == TF_BF16) return ce_fwd_launch<bf16>(st, rows, V, logits, ld, labels, loss, lse);
+  if (dtype == TF_F16) return ce_fwd_launch<f16>(st, rows, V, logits, map, labels, loss, lse);
+  if (dtype == TF_BF16) return ce_fwd_launch<bf16>(st, rows, V, logits, map, labels, loss, lse);
   return TF_EDTYPE;
 }
 
 extern "C" int tf_cross_entropy_bwd(void* stream, int dtype, int64_t rows, int64_t V, const void* logits,
-                                    int64_t ld, const int64_t* labels, const float* lse, const void* gout,
-                                    int64_t gout_stride, void* dlogits, int64_t ldd) {
+                                    int64_t ld, int64_t inner_rows, int64_t outer_stride, const int64_t* labels,
+                                    const float* lse, const void* gout, int64_t gout_stride, void* dlogits,
+                                    int64_t ldd, int64_t outer_stride_d) {
   if (!logits || !labels || !lse || !gout || !dlogits) return TF_EINVAL;
-  if (rows < 0 || rows > 0x7fffffff || V <= 0 || V > (1 << 30) || ld < V || ldd < V || gout_stride < 0)
-    return TF_EINVAL;
+  if (rows < 0 || rows > 0x7fffffff || V <= 0 || V > (1 << 30) || gout_stride < 0) return TF_EINVAL;
+  RowMap map, dmap;
+  if (!make_map(map, rows, V, ld, inner_rows, outer_stride)) return TF_EINVAL;
+  if (!make_map(dmap, rows, V, ldd, inner_rows, outer_stride_d)) return TF_EINVAL;
   if (rows == 0) return TF_OK;
   hipStream_t st = (hipStream_t)stream;
   if (dtype == TF_F16)
-    return ce_bwd_launch<f16>(st, rows, V, logits, ld, labels, lse, gout, gout_stride, dlogits, ldd);
+    return ce_bwd_launch<f16>(st, rows, V, logits, map, labels, lse, gout, gout_stride, dlogits, dmap);
   if (dtype == TF_BF16)
-    return ce_bwd_launch<bf16>(st, rows, V, logits, ld, labels, lse, gout, gout_stride, dlogits, ldd);
+    return ce_bwd_launch<bf16>(st, rows, V, logits, map, labels, lse, gout, gout_stride, dlogits, dmap);
   return TF_EDTYPE;
 }

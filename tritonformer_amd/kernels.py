@@ -280,16 +280,20 @@ def softmax_bwd(grad_out, saved_out):
 
 
 # --------------------------------------------------------------------------- cross entropy
-def cross_entropy_fwd(logits, labels):
-    """-> (per-row loss in logits' dtype, lse fp32); reference
-    kernels/crossentropy.py:47-75 (which keeps the full (N, V) matrix instead)."""
-    if logits.ndim != 2 or labels.ndim != 1 or labels.shape[0] != logits.shape[0]:
-        raise ValueError("cross entropy takes (N, V) logits and (N,) labels")
+def _check_ce(logits, labels):
     if labels.dtype != torch.int64:
         raise TypeError("labels must be int64")
     if logits.dtype not in (torch.float16, torch.bfloat16):
         raise TypeError("logits must be float16 or bfloat16")
     require_cuda(logits, labels)
+
+
+def cross_entropy_fwd(logits, labels):
+    """-> (per-row loss in logits' dtype, lse fp32, logits, labels); reference
+    kernels/crossentropy.py:47-75 (which keeps the full (N, V) matrix instead)."""
+    if logits.ndim != 2 or labels.ndim != 1 or labels.shape[0] != logits.shape[0]:
+        raise ValueError("cross entropy takes (N, V) logits and (N,) labels")
+    _check_ce(logits, labels)
     if logits.stride(-1) != 1:
         logits = logits.contiguous()
     labels = labels.contiguous()
@@ -297,7 +301,7 @@ def cross_entropy_fwd(logits, labels):
     loss = torch.empty((n,), dtype=logits.dtype, device=logits.device)
     lse = torch.empty((n,), dtype=torch.float32, device=logits.device)
     check(load().tf_cross_entropy_fwd(stream_ptr(), dtype_code(logits.dtype), n, v, logits.data_ptr(),
-                                      logits.stride(0), labels.data_ptr(), loss.data_ptr(), lse.data_ptr()))
+                                      logits.stride(0), 0, 0, labels.data_ptr(), loss.data_ptr(), lse.data_ptr()))
     return loss, lse, logits, labels
 
 
@@ -310,6 +314,42 @@ def cross_entropy_bwd(grad_out, logits, labels, lse):
     gstride = grad_out.stride(0) if grad_out.ndim == 1 else 0
     dlogits = torch.empty((n, v), dtype=logits.dtype, device=logits.device)
     check(load().tf_cross_entropy_bwd(stream_ptr(), dtype_code(logits.dtype), n, v, logits.data_ptr(),
-                                      logits.stride(0), labels.data_ptr(), lse.data_ptr(), grad_out.data_ptr(),
-                                      gstride, dlogits.data_ptr(), v))
+                                      logits.stride(0), 0, 0, labels.data_ptr(), lse.data_ptr(),
+                                      grad_out.data_ptr(), gstride, dlogits.data_ptr(), v, 0))
+    return dlogits
+
+
+def shifted_cross_entropy_fwd(logits, labels):
+    """Next-token loss of a (B, S, V) logits tensor against (B, S) labels:
+    row (b, s), s < S-1, is scored against labels[b, s+1], reading the logits in
+    place (the reference copies logits[..., :-1, :] first, transformer.py:333-334).
+    -> (loss (B*(S-1),), lse, logits, shifted labels)"""
+    if logits.ndim != 3 or labels.shape != logits.shape[:2]:
+        raise ValueError("shifted cross entropy takes (B, S, V) logits and (B, S) labels")
+    _check_ce(logits, labels)
+    if not logits.is_contiguous():
+        logits = logits.contiguous()
+    b, s, v = logits.shape
+    shift_labels = labels[:, 1:].contiguous().view(-1)
+    n = b * (s - 1)
+    loss = torch.empty((n,), dtype=logits.dtype, device=logits.device)
+    lse = torch.empty((n,), dtype=torch.float32, device=logits.device)
+    check(load().tf_cross_entropy_fwd(stream_ptr(), dtype_code(logits.dtype), n, v, logits.data_ptr(), v, s - 1,
+                                      s * v, shift_labels.data_ptr(), loss.data_ptr(), lse.data_ptr()))
+    return loss, lse, logits, shift_labels
+
+
+def shifted_cross_entropy_bwd(grad_out, logits, shift_labels, lse):
+    """Gradient with respect to the full (B, S, V) logits: rows s < S-1 as
+    cross_entropy_bwd, the last position of every sequence zero."""
+    b, s, v = logits.shape
+    n = b * (s - 1)
+    if grad_out.dtype != logits.dtype:
+        grad_out = grad_out.to(logits.dtype)
+    gstride = grad_out.stride(0) if grad_out.ndim == 1 else 0
+    dlogits = torch.empty((b, s, v), dtype=logits.dtype, device=logits.device)
+    dlogits[:, -1].zero_()
+    check(load().tf_cross_entropy_bwd(stream_ptr(), dtype_code(logits.dtype), n, v, logits.data_ptr(), v, s - 1,
+                                      s * v, shift_labels.data_ptr(), lse.data_ptr(), grad_out.data_ptr(), gstride,
+                                      dlogits.data_ptr(), v, s * v))
     return dlogits

@@ -18,7 +18,7 @@ from typing import List, Optional, Tuple
 import torch
 import torch.nn as nn
 
-from . import cross_entropy_loss, fast_causal_attention, fast_causal_attention_with_bias
+from . import fast_causal_attention, fast_causal_attention_with_bias, shifted_cross_entropy_loss
 from . import nn as tnn
 
 
@@ -191,7 +191,7 @@ class Transformer(nn.Module):
         logits_lm = self.logits_out(hidden_states)
         if labels is None:
             return logits_lm
-        shift_logits = logits_lm[..., :-1, :].contiguous()
-        shift_labels = labels[..., 1:].contiguous()
-        loss = cross_entropy_loss.apply(shift_logits.view(-1, shift_logits.size(-1)), shift_labels.view(-1))
+        # same rows and labels as the reference's shift-copy-then-cross-entropy
+        # (transformer.py:333-341), read from logits_lm in place
+        loss = shifted_cross_entropy_loss.apply(logits_lm, labels)
         return logits_lm, loss.mean()
