@@ -90,9 +90,11 @@ int tf_gemm_tune(int cfg, int splits);
  * result write-out (WRONG results: it exists to time the main loop alone). */
 int tf_gemm_debug_flags(int flags);
 
-/* Causal flash attention forward.  q,k,v,o: logical (B, nh, S, hd) with the
- * SAME element strides {sb, sh, ss} and unit stride along hd (the reference
- * passes q's strides for all four, kernels/attention.py:202-205).
+/* Causal flash attention forward.  q, k, v: logical (B, nh, S, hd) sharing the
+ * element strides {sb, sh, ss}; o: the same logical shape with its own strides
+ * {osb, osh, oss}; unit stride along hd everywhere.  (The reference passes q's
+ * strides for all four, kernels/attention.py:202-205; separate output strides
+ * also serve q, k, v that are slices of one packed (B, S, 3, nh, hd) buffer.)
  * lse: (B, nh, S) fp32, contiguous, log2-domain log-sum-exp of the scaled
  * (and biased) scores.  bias: NULL, or (nh, Sb, Sb) with Sb >= S, element
  * strides {bias_sh, bias_sr}, unit stride along keys, added after scaling
@@ -102,19 +104,20 @@ int tf_gemm_debug_flags(int flags);
  * Preconditions (as the reference asserts): hd in {32,64,128}; S % 64 == 0. */
 int tf_attn_fwd(void* stream, int dtype, int64_t B, int64_t nh, int64_t S, int64_t hd,
                 const void* q, const void* k, const void* v, void* o,
-                int64_t sb, int64_t sh, int64_t ss,
+                int64_t sb, int64_t sh, int64_t ss, int64_t osb, int64_t osh, int64_t oss,
                 float* lse, const void* bias, int64_t bias_sh, int64_t bias_sr,
                 float scale);
 
-/* Backward of the above: dq, dk, dv have q's strides.  delta: (B, nh, S) fp32
- * scratch (row sums of dO*O), written then read by this call.
+/* Backward of the above: dq, dk, dv have q's strides, o and d_o the output
+ * strides.  delta: (B, nh, S) fp32 scratch (row sums of dO*O), written then read
+ * by this call.
  * Replaces flash_wrapper_bwd (kernels/attention.py:550-607) and
  * flash_wrapper_bwd_attn_bias (kernels/biased_attention.py:598-660).
  * No gradient is produced for the bias (tritonformer/attention.py:60). */
 int tf_attn_bwd(void* stream, int dtype, int64_t B, int64_t nh, int64_t S, int64_t hd,
                 const void* q, const void* k, const void* v, const void* o, const void* d_o,
                 void* dq, void* dk, void* dv,
-                int64_t sb, int64_t sh, int64_t ss,
+                int64_t sb, int64_t sh, int64_t ss, int64_t osb, int64_t osh, int64_t oss,
                 const float* lse, float* delta,
                 const void* bias, int64_t bias_sh, int64_t bias_sr, float scale);
 

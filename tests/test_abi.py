@@ -73,8 +73,9 @@ def test_attention_rejects_bad_shapes():
 
     def fwd(S, hd, ss=None, dtype=0, bias=None, bsr=0):
         ss = ss if ss is not None else hd
-        return lib.tf_attn_fwd(None, dtype, 1, 2, S, hd, FAKE, FAKE, FAKE, FAKE, S * 2 * hd, hd, 2 * hd if ss == hd else ss,
-                               FAKE, bias, bsr * bsr if bias else 0, bsr, 0.125)
+        row = 2 * hd if ss == hd else ss
+        return lib.tf_attn_fwd(None, dtype, 1, 2, S, hd, FAKE, FAKE, FAKE, FAKE, S * 2 * hd, hd, row, S * 2 * hd, hd,
+                               2 * hd, FAKE, bias, bsr * bsr if bias else 0, bsr, 0.125)
 
     assert fwd(100, 64) == -4           # S % 64 != 0
     assert fwd(128, 48) == -4           # head_dim not in {32, 64, 128}
@@ -82,7 +83,7 @@ def test_attention_rejects_bad_shapes():
     assert fwd(128, 64, ss=60) == -3    # row stride not a multiple of 8 elements
     assert fwd(128, 64, bias=FAKE, bsr=64) == -3   # bias rows shorter than S
     assert lib.tf_attn_bwd(None, 0, 1, 2, 128, 64, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, None, 16384, 64, 128,
-                           FAKE, FAKE, None, 0, 0, 0.125) == -1  # null dv
+                           16384, 64, 128, FAKE, FAKE, None, 0, 0, 0.125) == -1  # null dv
 
 
 def test_row_kernels_reject_bad_arguments():

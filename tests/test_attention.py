@@ -124,3 +124,29 @@ def test_baseline_config_shapes(dims, dev):
         assert_close(o[bi:bi + 1], orf, name="o")
         for got, ref, nm in zip(grads, (qr, kr, vr), "qkv"):
             assert_close(got[bi:bi + 1], ref.grad, name="d" + nm)
+
+
+@pytest.mark.parametrize("use_bias", [False, True])
+def test_packed_qkv_equals_three_slices(use_bias, dev):
+    """The packed Function runs the same kernels on strided slices of one buffer:
+    results must equal the three-tensor Function bit for bit, gradient included."""
+    b, s, nh, hd = 2, 256, 4, 64
+    g = torch.Generator().manual_seed(11)
+    qkv = torch.randn(b, s, 3, nh, hd, generator=g).half().to(dev)
+    do = torch.randn(b, s, nh * hd, generator=g).half().to(dev)
+    bias = R.alibi_mask(s, nh).to(dev) if use_bias else None
+    a = qkv.clone().requires_grad_(True)
+    out_p = T.fast_causal_attention_qkvpacked.apply(a, bias)
+    out_p.backward(do)
+    parts = [qkv[:, :, i].permute(0, 2, 1, 3).contiguous().requires_grad_(True) for i in range(3)]
+    if use_bias:
+        out_s = T.fast_causal_attention_with_bias.apply(*parts, bias)
+    else:
+        out_s = T.fast_causal_attention.apply(*parts)
+    out_s.backward(do.view(b, s, nh, hd).permute(0, 2, 1, 3))
+    assert out_p.shape == (b, s, nh * hd)
+    assert torch.equal(out_p.view(b, s, nh, hd).permute(0, 2, 1, 3), out_s)
+    for i in range(3):
+        assert torch.equal(a.grad[:, :, i].permute(0, 2, 1, 3), parts[i].grad)
+    o_ref = R.causal_attention(*[p_.detach().cpu() for p_ in parts], bias.cpu() if use_bias else None)
+    assert_close(out_s, o_ref, name="packed vs oracle")

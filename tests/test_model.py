@@ -105,3 +105,27 @@ def test_step_is_deterministic(dev):
         loss.backward()
         outs.append((loss.item(), model.layer_list[0].attention.q_proj.weight.grad.clone()))
     assert outs[0][0] == outs[1][0] and torch.equal(outs[0][1], outs[1][1])
+
+
+def test_unfused_reference_path_matches_fused(dev):
+    """FUSE_QKV=False runs the three projections exactly as the reference module
+    does; both paths must agree (same kernels, same per-element arithmetic)."""
+    import tritonformer_amd.transformer as tr
+
+    cfg, ref, ids = build_config1()
+    model = Transformer(to_cfg(cfg), device=dev, param_dtype=torch.float32)
+    model.load_state_dict(ref.state_dict())
+    results = []
+    for fuse in (True, False):
+        tr.FUSE_QKV = fuse
+        try:
+            model.zero_grad(set_to_none=True)
+            with torch.autocast("cuda", dtype=torch.float16):
+                _, loss = model(ids.to(dev), ids.to(dev))
+            (loss * LOSS_SCALE).backward()
+            results.append((loss.item(), {n: p.grad.clone() for n, p in model.named_parameters()}))
+        finally:
+            tr.FUSE_QKV = True
+    assert abs(results[0][0] - results[1][0]) <= 1e-3 * abs(results[1][0])
+    for n in results[0][1]:
+        assert rel_l2(results[0][1][n], results[1][1][n]) < 2e-2, n

@@ -5,6 +5,7 @@ exports, backed by hand-written HIP kernels behind a C ABI."""
 # not been built that call raises: there is no PyTorch or CPU fallback.
 from .attention import BiasedCausalAttention as fast_causal_attention_with_bias
 from .attention import CausalAttention as fast_causal_attention
+from .attention import PackedCausalAttention as fast_causal_attention_qkvpacked
 from .crossentropy import CrossEntropyLoss as cross_entropy_loss
 from .crossentropy import ShiftedCrossEntropyLoss as shifted_cross_entropy_loss
 from .layernorm import LayerNorm as layer_norm

@@ -26,9 +26,10 @@ SIGNATURES = {
     "tf_gemm_workspace_bytes": (_i64, [_i, _i, _i64, _i64, _i64]),
     "tf_gemm_tune": (_i, [_i, _i]),
     "tf_gemm_debug_flags": (_i, [_i]),
-    "tf_attn_fwd": (_i, [_vp, _i, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _i64, _f]),
+    "tf_attn_fwd": (_i, [_vp, _i, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64,
+                         _vp, _vp, _i64, _i64, _f]),
     "tf_attn_bwd": (_i, [_vp, _i, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64,
-                         _vp, _vp, _vp, _i64, _i64, _f]),
+                         _i64, _i64, _i64, _vp, _vp, _vp, _i64, _i64, _f]),
     "tf_layernorm_fwd": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _vp, _vp, _f, _vp, _i64, _vp, _vp]),
     "tf_layernorm_bwd": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _i64]),
     "tf_layernorm_bwd_partial_bytes": (_i64, [_i64, _i64]),

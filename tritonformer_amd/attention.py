@@ -48,3 +48,39 @@ class BiasedCausalAttention(Function):
         lse, query, key, value, out, attn_bias = ctx.saved_tensors
         dq, dk, dv = flash_wrapper_bwd_attn_bias(grad_output, out, query, key, value, lse, attn_bias)
         return dq, dk, dv, None
+
+
+class PackedCausalAttention(Function):
+    """Causal attention on a packed projection: ``apply(qkv, attn_bias_or_None)``
+    with qkv (B, S, 3, nh, hd) -- the output of ONE (d, 3d) GEMM -- returns
+    (B, S, nh*hd); the backward writes dq, dk, dv straight into one packed
+    (B, S, 3, nh, hd) gradient, so the projection's dX and dW are single GEMMs
+    too.  Same kernels as CausalAttention / BiasedCausalAttention, which take the
+    three strided slices as they are.  No counterpart in the reference (three
+    separate projections, transformer.py:158-175)."""
+
+    @staticmethod
+    @amp_fwd
+    def forward(ctx: Any, qkv: torch.Tensor, attn_bias) -> torch.Tensor:
+        if qkv.ndim != 5 or qkv.shape[2] != 3:
+            raise ValueError("packed attention takes qkv of shape (B, S, 3, nh, hd)")
+        if not qkv.is_contiguous():
+            qkv = qkv.contiguous()
+        b, s, _, nh, hd = qkv.shape
+        q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+        out = torch.empty((b, s, nh, hd), dtype=qkv.dtype, device=qkv.device)
+        _, lse = flash_wrapper_fwd(q, k, v, attn_bias, out=out.permute(0, 2, 1, 3))
+        ctx.save_for_backward(lse, qkv, out, attn_bias)
+        return out.view(b, s, nh * hd)
+
+    @staticmethod
+    @amp_bwd
+    def backward(ctx: Any, grad_output: torch.Tensor):
+        lse, qkv, out, attn_bias = ctx.saved_tensors
+        b, s, _, nh, hd = qkv.shape
+        q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+        dqkv = torch.empty_like(qkv)
+        grads = tuple(dqkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+        grad_output = grad_output.reshape(b, s, nh, hd).permute(0, 2, 1, 3)
+        flash_wrapper_bwd(grad_output, out.permute(0, 2, 1, 3), q, k, v, lse, attn_bias, grads=grads)
+        return dqkv, None

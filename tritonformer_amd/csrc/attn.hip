@@ -30,7 +30,8 @@ struct AttnParams {
   float* lse;    // written by fwd, read by bwd
   float* delta;  // written by the bwd pre-pass
   const void* bias;
-  int64_t sb, sh, ss;         // element strides of q/k/v/o and their grads
+  int64_t sb, sh, ss;         // element strides of q, k, v and of dq, dk, dv
+  int64_t osb, osh, oss;      // element strides of o and dO
   int64_t bias_sh, bias_sr;   // element strides of bias (head, query row)
   int B, nh, S;
   float scale_log2;           // scale * log2(e)
@@ -139,7 +140,7 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_fw
   const T* Q = (const T*)p.q + base;
   const T* K = (const T*)p.k + base;
   const T* V = (const T*)p.v + base;
-  T* O = (T*)p.out + base;
+  T* O = (T*)p.out + (int64_t)b * p.osb + (int64_t)h * p.osh;
 
   const int q0 = qblk * 128;
   const int q0w = q0 + wave * 32;
@@ -276,7 +277,7 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_fw
         v4 o;
 #pragma unroll
         for (int e = 0; e < 4; ++e) o[e] = (T)(oacc[d][g * 4 + e] * inv);
-        *reinterpret_cast<v4*>(O + (int64_t)myq * p.ss + d * 32 + g * 8 + 4 * (lane >> 5)) = o;
+        *reinterpret_cast<v4*>(O + (int64_t)myq * p.oss + d * 32 + g * 8 + 4 * (lane >> 5)) = o;
       }
   }
 }
@@ -292,7 +293,7 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(AttnParams p) {
   const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / LPR;  // over nbh * S
   if (row >= (int64_t)nbh * p.S) return;
   const int bh = (int)(row / p.S), s = (int)(row % p.S);
-  const int64_t off = (int64_t)(bh / p.nh) * p.sb + (int64_t)(bh % p.nh) * p.sh + (int64_t)s * p.ss +
+  const int64_t off = (int64_t)(bh / p.nh) * p.osb + (int64_t)(bh % p.nh) * p.osh + (int64_t)s * p.oss +
                       (threadIdx.x % LPR) * 8;
   float a[8], g[8];
   Chunk<T>::load((const T*)p.o + off, a);
@@ -327,7 +328,7 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_dkdv_kernel(AttnPa
   const T* Q = (const T*)p.q + base;
   const T* K = (const T*)p.k + base;
   const T* V = (const T*)p.v + base;
-  const T* dO = (const T*)p.d_o + base;
+  const T* dO = (const T*)p.d_o + (int64_t)b * p.osb + (int64_t)h * p.osh;
   const float* lse = p.lse + (int64_t)bh * p.S;
   const float* delta = p.delta + (int64_t)bh * p.S;
 
@@ -359,7 +360,7 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_dkdv_kernel(AttnPa
 
   auto fetch = [&](int qb) {
     QT::fetch(rq, Q, p.ss, qb);
-    QT::fetch(rdo, dO, p.ss, qb);
+    QT::fetch(rdo, dO, p.oss, qb);
     if (threadIdx.x < 64) rstat = -lse[qb + threadIdx.x];
     else if (threadIdx.x < 128) rstat = -delta[qb + threadIdx.x - 64];
   };
@@ -477,7 +478,7 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_dq
   const T* Q = (const T*)p.q + base;
   const T* K = (const T*)p.k + base;
   const T* V = (const T*)p.v + base;
-  const T* dO = (const T*)p.d_o + base;
+  const T* dO = (const T*)p.d_o + (int64_t)b * p.osb + (int64_t)h * p.osh;
 
   const int q0 = qblk * 128;
   const int q0w = q0 + wave * 32;
@@ -493,7 +494,7 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_dq
     u32x4 a = {0u, 0u, 0u, 0u}, c = {0u, 0u, 0u, 0u};
     if (active) {
       a = ld16(Q + (int64_t)myq * p.ss + ks * 16 + (lane >> 5) * 8);
-      c = ld16(dO + (int64_t)myq * p.ss + ks * 16 + (lane >> 5) * 8);
+      c = ld16(dO + (int64_t)myq * p.oss + ks * 16 + (lane >> 5) * 8);
     }
     qf[ks] = __builtin_bit_cast(v8, a);
     dof[ks] = __builtin_bit_cast(v8, c);
@@ -653,13 +654,14 @@ static int attn_dispatch(hipStream_t st, int hd, bool has_bias, const AttnParams
 }
 
 static int attn_check(int dtype, int64_t B, int64_t nh, int64_t S, int64_t hd, int64_t sb, int64_t sh, int64_t ss,
-                      const void* bias, int64_t bias_sh, int64_t bias_sr) {
+                      int64_t osb, int64_t osh, int64_t oss, const void* bias, int64_t bias_sh, int64_t bias_sr) {
   if (dtype != TF_F16 && dtype != TF_BF16) return TF_EDTYPE;
   if (B <= 0 || nh <= 0 || S <= 0) return TF_EINVAL;
   if (hd != 32 && hd != 64 && hd != 128) return TF_ESHAPE;  // as kernels/attention.py:567
   if (S % 64 != 0) return TF_ESHAPE;                        // as kernels/attention.py:181-183
   if (B * nh * ((S + 127) / 128) > 0x7fffffff || S > (1 << 24)) return TF_EINVAL;
   if (sb % 8 || sh % 8 || ss % 8 || ss < hd) return TF_EALIGN;
+  if (osb % 8 || osh % 8 || oss % 8 || oss < hd) return TF_EALIGN;
   if (bias && (bias_sh % 4 || bias_sr % 4 || bias_sr < S)) return TF_EALIGN;
   return TF_OK;
 }
@@ -669,16 +671,18 @@ static int attn_check(int dtype, int64_t B, int64_t nh, int64_t S, int64_t hd, i
 using namespace tfa;
 
 extern "C" int tf_attn_fwd(void* stream, int dtype, int64_t B, int64_t nh, int64_t S, int64_t hd, const void* q,
-                           const void* k, const void* v, void* o, int64_t sb, int64_t sh, int64_t ss, float* lse,
-                           const void* bias, int64_t bias_sh, int64_t bias_sr, float scale) {
+                           const void* k, const void* v, void* o, int64_t sb, int64_t sh, int64_t ss, int64_t osb,
+                           int64_t osh, int64_t oss, float* lse, const void* bias, int64_t bias_sh, int64_t bias_sr,
+                           float scale) {
   if (!q || !k || !v || !o || !lse) return TF_EINVAL;
-  const int rc = attn_check(dtype, B, nh, S, hd, sb, sh, ss, bias, bias_sh, bias_sr);
+  const int rc = attn_check(dtype, B, nh, S, hd, sb, sh, ss, osb, osh, oss, bias, bias_sh, bias_sr);
   if (rc != TF_OK) return rc;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o)) return TF_EALIGN;
   if (bias && (reinterpret_cast<uintptr_t>(bias) & 7)) return TF_EALIGN;
   AttnParams p = {};
   p.q = q; p.k = k; p.v = v; p.out = o; p.lse = lse; p.bias = bias;
-  p.sb = sb; p.sh = sh; p.ss = ss; p.bias_sh = bias_sh; p.bias_sr = bias_sr;
+  p.sb = sb; p.sh = sh; p.ss = ss; p.osb = osb; p.osh = osh; p.oss = oss;
+  p.bias_sh = bias_sh; p.bias_sr = bias_sr;
   p.B = (int)B; p.nh = (int)nh; p.S = (int)S;
   p.scale = scale; p.scale_log2 = scale * kLog2e;
   hipStream_t st = (hipStream_t)stream;
@@ -688,10 +692,11 @@ extern "C" int tf_attn_fwd(void* stream, int dtype, int64_t B, int64_t nh, int64
 
 extern "C" int tf_attn_bwd(void* stream, int dtype, int64_t B, int64_t nh, int64_t S, int64_t hd, const void* q,
                            const void* k, const void* v, const void* o, const void* d_o, void* dq, void* dk, void* dv,
-                           int64_t sb, int64_t sh, int64_t ss, const float* lse, float* delta, const void* bias,
-                           int64_t bias_sh, int64_t bias_sr, float scale) {
+                           int64_t sb, int64_t sh, int64_t ss, int64_t osb, int64_t osh, int64_t oss,
+                           const float* lse, float* delta, const void* bias, int64_t bias_sh, int64_t bias_sr,
+                           float scale) {
   if (!q || !k || !v || !o || !d_o || !dq || !dk || !dv || !lse || !delta) return TF_EINVAL;
-  const int rc = attn_check(dtype, B, nh, S, hd, sb, sh, ss, bias, bias_sh, bias_sr);
+  const int rc = attn_check(dtype, B, nh, S, hd, sb, sh, ss, osb, osh, oss, bias, bias_sh, bias_sr);
   if (rc != TF_OK) return rc;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o) || !aligned16(d_o) || !aligned16(dq) ||
       !aligned16(dk) || !aligned16(dv))
@@ -700,7 +705,8 @@ extern "C" int tf_attn_bwd(void* stream, int dtype, int64_t B, int64_t nh, int64
   AttnParams p = {};
   p.q = q; p.k = k; p.v = v; p.o = o; p.d_o = d_o; p.dq = dq; p.dk = dk; p.dv = dv;
   p.lse = const_cast<float*>(lse); p.delta = delta; p.bias = bias;
-  p.sb = sb; p.sh = sh; p.ss = ss; p.bias_sh = bias_sh; p.bias_sr = bias_sr;
+  p.sb = sb; p.sh = sh; p.ss = ss; p.osb = osb; p.osh = osh; p.oss = oss;
+  p.bias_sh = bias_sh; p.bias_sr = bias_sr;
   p.B = (int)B; p.nh = (int)nh; p.S = (int)S;
   p.scale = scale; p.scale_log2 = scale * kLog2e;
   hipStream_t st = (hipStream_t)stream;

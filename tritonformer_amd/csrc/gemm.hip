@@ -647,35 +647,30 @@ static int g_force_cfg = env_int("TF_GEMM_CFG", -1);
 static int g_force_splits = env_int("TF_GEMM_SPLITS", 0);
 static int g_flags = env_int("TF_GEMM_FLAGS", 0);
 
-static GemmPlan make_plan(int64_t M, int64_t N, int64_t K, bool vec) {
+// Tile shape, contraction split and the rough cost (microseconds) of running
+// M x N x K with tile configuration `cfg`.  The cost constants are fits to
+// rocprofv3 kernel durations on MI355X: one "round" of workgroups (one per CU)
+// costs a fixed part (launch, cold first loads, result write-out) plus a part
+// per 64-wide contraction step.
+static GemmPlan plan_for(int cfg, int64_t M, int64_t N, int64_t K, double* cost_us) {
   GemmPlan pl;
-  const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
-  // Measured on MI355X (gfx950): 256x256 tiles win once they alone give every CU
-  // work, and for long contractions over a mid-sized output (weight gradients of
-  // the MLP) when combined with a contraction split; smaller outputs run 256x128
-  // tiles (one workgroup of eight waves per CU), very long contractions over a small
-  // output 128x128 tiles with two workgroups resident per CU.
-  const bool dma = vec && K % 64 == 0;
-  const bool long_k_mid = big_tiles >= 48 && big_tiles < 128 && K >= 4096 && K >= 2 * (M > N ? M : N);
-  if (big_tiles >= 200 || long_k_mid) pl.cfg = dma ? 2 : 0;
-  else if (dma) pl.cfg = K >= 16384 ? 3 : 4;
-  else pl.cfg = 1;
-  if (g_force_cfg >= 0 && g_force_cfg < kNumCfgs) pl.cfg = g_force_cfg;
-  if (kCfgs[pl.cfg].dma && !(vec && K % kCfgs[pl.cfg].bk == 0))
-    pl.cfg = kCfgs[pl.cfg].bm * kCfgs[pl.cfg].bn >= 256 * 256 ? 0 : 1;  // register-staged twin
-  pl.bm = kCfgs[pl.cfg].bm;
-  pl.bn = kCfgs[pl.cfg].bn;
-  pl.bk = kCfgs[pl.cfg].bk;
+  pl.cfg = cfg;
+  pl.bm = kCfgs[cfg].bm;
+  pl.bn = kCfgs[cfg].bn;
+  pl.bk = kCfgs[cfg].bk;
   pl.tiles_m = (int)((M + pl.bm - 1) / pl.bm);
   pl.tiles_n = (int)((N + pl.bn - 1) / pl.bn);
   const int64_t tiles = (int64_t)pl.tiles_m * pl.tiles_n;
   const int64_t ksteps = (K + pl.bk - 1) / pl.bk;
+  const int wg_per_cu = pl.bm * pl.bn <= 128 * 128 ? 2 : 1;
+  const int64_t slots = 256 * wg_per_cu;
   // Split the contraction only when the tiles alone leave most CUs idle (weight
-  // gradients of square layers: few output tiles, long contraction); every slice
-  // keeps at least 16 steps so the fp32 partial traffic stays small.
+  // gradients: few output tiles, long contraction); never beyond one full round of
+  // workgroups, and every slice keeps at least 16 steps so that the fp32 partial
+  // traffic stays small.
   int64_t splits = 1;
-  if (tiles < 128) {
-    splits = (256 + tiles - 1) / tiles;
+  if (tiles <= slots / 2) {
+    splits = slots / tiles;
     const int64_t max_by_k = ksteps / 16 > 0 ? ksteps / 16 : 1;
     if (splits > max_by_k) splits = max_by_k;
     if (splits > 16) splits = 16;
@@ -686,7 +681,38 @@ static GemmPlan make_plan(int64_t M, int64_t N, int64_t K, bool vec) {
   pl.k_per_split = (int)(steps_per * pl.bk);
   pl.splits = (int)((ksteps + steps_per - 1) / steps_per);
   if (pl.splits < 1) pl.splits = 1;
+  if (cost_us) {
+    const double fixed = pl.bm * pl.bn >= 256 * 256 ? 10.0 : 7.0;
+    const double per_step = pl.bm * pl.bn >= 256 * 256 ? 1.65 : (pl.bm * pl.bn >= 256 * 128 ? 1.15 : 1.1);
+    const int64_t rounds = (tiles * pl.splits + slots - 1) / slots;
+    double c = (double)rounds * (fixed + per_step * (double)steps_per);
+    if (pl.splits > 1) c += 3.0 + (pl.splits + 0.5) * (double)M * (double)N * 4.0 / 5.0e6;
+    *cost_us = c;
+  }
   return pl;
+}
+
+static GemmPlan make_plan(int64_t M, int64_t N, int64_t K, bool vec) {
+  const bool dma = vec && K % 64 == 0;
+  if (g_force_cfg >= 0 && g_force_cfg < kNumCfgs) {
+    int cfg = g_force_cfg;
+    if (kCfgs[cfg].dma && !dma) cfg = kCfgs[cfg].bm * kCfgs[cfg].bn >= 256 * 256 ? 0 : 1;  // register-staged twin
+    return plan_for(cfg, M, N, K, nullptr);
+  }
+  // candidates: 256x256 and 256x128 / 128x128 tiles, direct-to-LDS kernels when their
+  // preconditions hold, the register-staged twins otherwise
+  const int cand_dma[3] = {2, 4, 3};
+  const int cand_reg[2] = {0, 1};
+  const int* cand = dma ? cand_dma : cand_reg;
+  const int ncand = dma ? 3 : 2;
+  GemmPlan best = plan_for(cand[0], M, N, K, nullptr);
+  double best_cost = 1e30;
+  for (int i = 0; i < ncand; ++i) {
+    double c;
+    const GemmPlan pl = plan_for(cand[i], M, N, K, &c);
+    if (c < best_cost) { best_cost = c; best = pl; }
+  }
+  return best;
 }
 
 template <typename K>

@@ -162,43 +162,55 @@ def _bias_args(bias):
     return bias, bias.data_ptr(), bias.stride(0), bias.stride(1)
 
 
-def flash_wrapper_fwd(q, k, v, bias=None):
-    """Causal attention forward -> (out, lse).  ``out`` has q's strides; ``lse``
-    is (B, nh, S) fp32 in the log2 domain (the reference keeps fp16 m and l,
-    kernels/attention.py:171-217 and kernels/biased_attention.py:188-245)."""
+def _strided_ok(t):
+    return t.stride(-1) == 1 and all(st % 8 == 0 for st in t.stride()[:-1]) and t.data_ptr() % 16 == 0
+
+
+def flash_wrapper_fwd(q, k, v, bias=None, out=None):
+    """Causal attention forward -> (out, lse).  ``out`` has q's strides unless a
+    (B, nh, S, hd) view is passed in; ``lse`` is (B, nh, S) fp32 in the log2
+    domain (the reference keeps fp16 m and l, kernels/attention.py:171-217 and
+    kernels/biased_attention.py:188-245)."""
     _check_attn(q, k, v, bias)
     q, k, v = _attn_layout(q, k, v)
     b, nh, s, hd = q.shape
-    out = torch.empty_like(q)
-    if out.stride() != q.stride():
+    if out is None:
         out = torch.empty_strided(q.shape, q.stride(), dtype=q.dtype, device=q.device)
+    elif out.shape != q.shape or out.dtype != q.dtype or not _strided_ok(out):
+        raise ValueError("attention output buffer must match q in shape and dtype, with aligned strides")
     lse = torch.empty((b, nh, s), dtype=torch.float32, device=q.device)
     bias, bptr, bsh, bsr = _bias_args(bias)
     check(load().tf_attn_fwd(stream_ptr(), dtype_code(q.dtype), b, nh, s, hd, q.data_ptr(), k.data_ptr(),
-                             v.data_ptr(), out.data_ptr(), q.stride(0), q.stride(1), q.stride(2), lse.data_ptr(),
-                             bptr, bsh, bsr, 1.0 / math.sqrt(hd)))
+                             v.data_ptr(), out.data_ptr(), q.stride(0), q.stride(1), q.stride(2), out.stride(0),
+                             out.stride(1), out.stride(2), lse.data_ptr(), bptr, bsh, bsr, 1.0 / math.sqrt(hd)))
     return out, lse
 
 
-def flash_wrapper_bwd(grad_out, out, q, k, v, lse, bias=None):
-    """Causal attention backward -> (dq, dk, dv), each with q's strides
-    (reference kernels/attention.py:550-607, kernels/biased_attention.py:598-660)."""
+def flash_wrapper_bwd(grad_out, out, q, k, v, lse, bias=None, grads=None):
+    """Causal attention backward -> (dq, dk, dv), each with q's strides (or written
+    into the three (B, nh, S, hd) views given as ``grads``); reference
+    kernels/attention.py:550-607, kernels/biased_attention.py:598-660."""
     _check_attn(q, k, v, bias)
-    q, k, v, out = _attn_layout(q, k, v, out)
-    if grad_out.stride() != q.stride() or grad_out.data_ptr() % 16:
-        g = torch.empty_strided(q.shape, q.stride(), dtype=q.dtype, device=q.device)
+    q, k, v = _attn_layout(q, k, v)
+    if not _strided_ok(out):
+        out = out.contiguous()
+    if grad_out.stride() != out.stride() or grad_out.data_ptr() % 16:
+        g = torch.empty_strided(out.shape, out.stride(), dtype=out.dtype, device=out.device)
         g.copy_(grad_out)
         grad_out = g
     b, nh, s, hd = q.shape
-    dq = torch.empty_strided(q.shape, q.stride(), dtype=q.dtype, device=q.device)
-    dk = torch.empty_strided(q.shape, q.stride(), dtype=q.dtype, device=q.device)
-    dv = torch.empty_strided(q.shape, q.stride(), dtype=q.dtype, device=q.device)
+    if grads is None:
+        grads = tuple(torch.empty_strided(q.shape, q.stride(), dtype=q.dtype, device=q.device) for _ in range(3))
+    dq, dk, dv = grads
+    if any(t.stride() != q.stride() or t.data_ptr() % 16 for t in grads):
+        raise ValueError("attention gradient buffers must share q's strides")
     delta = torch.empty((b, nh, s), dtype=torch.float32, device=q.device)
     bias, bptr, bsh, bsr = _bias_args(bias)
     check(load().tf_attn_bwd(stream_ptr(), dtype_code(q.dtype), b, nh, s, hd, q.data_ptr(), k.data_ptr(),
                              v.data_ptr(), out.data_ptr(), grad_out.data_ptr(), dq.data_ptr(), dk.data_ptr(),
-                             dv.data_ptr(), q.stride(0), q.stride(1), q.stride(2), lse.data_ptr(),
-                             delta.data_ptr(), bptr, bsh, bsr, 1.0 / math.sqrt(hd)))
+                             dv.data_ptr(), q.stride(0), q.stride(1), q.stride(2), out.stride(0), out.stride(1),
+                             out.stride(2), lse.data_ptr(), delta.data_ptr(), bptr, bsh, bsr,
+                             1.0 / math.sqrt(hd)))
     return dq, dk, dv
 
 

@@ -18,7 +18,13 @@ from typing import List, Optional, Tuple
 import torch
 import torch.nn as nn
 
-from . import fast_causal_attention, fast_causal_attention_with_bias, shifted_cross_entropy_loss
+from . import (
+    fast_causal_attention,
+    fast_causal_attention_qkvpacked,
+    fast_causal_attention_with_bias,
+    linear_no_bias,
+    shifted_cross_entropy_loss,
+)
 from . import nn as tnn
 
 
@@ -59,6 +65,12 @@ def generate_alibi_mask(seq_len: int, num_heads: int, device=None, dtype=torch.f
     bias = dist[None] * slopes[:, None, None]
     above = pos[None, :] > pos[:, None]
     return bias.masked_fill(above[None], float("-inf"))[None]
+
+
+# True: q/k/v projections run as one packed GEMM + packed attention (same parameters and
+# arithmetic per output element); False: three projections exactly as the reference
+# module does (transformer.py:158-182).
+FUSE_QKV = True
 
 
 def _weights_init(model: nn.Module, num_layers: int) -> None:
@@ -104,6 +116,13 @@ class CausalAttention(nn.Module):
 
     def forward(self, hidden_states: torch.Tensor, attn_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
         batch_size, q_seq_len, hidden_dim = hidden_states.shape
+        if FUSE_QKV:
+            # one (d, 3d) GEMM instead of three (d, d): same parameters, concatenated on the fly;
+            # autograd splits the weight gradient back into the three parameters
+            w_qkv = torch.cat([self.q_proj.weight, self.k_proj.weight, self.v_proj.weight], dim=1)
+            qkv = linear_no_bias.apply(hidden_states, w_qkv)
+            qkv = qkv.view(batch_size, q_seq_len, 3, self.num_attention_heads, self.hidden_size_per_attention_head)
+            return self.out_proj(fast_causal_attention_qkvpacked.apply(qkv, attn_bias))
         query_layer = self._heads(self.q_proj(hidden_states))
         key_layer = self._heads(self.k_proj(hidden_states))
         value_layer = self._heads(self.v_proj(hidden_states))
