@@ -126,8 +126,10 @@ int tf_attn_bwd(void* stream, int dtype, int64_t B, int64_t nh, int64_t S, int64
 /* y = gamma * (x - mean) * rstd + beta over the last dimension; biased
  * variance, rstd = 1/sqrt(var + eps), statistics in fp32
  * (kernels/layernorm.py:8-61, launcher :64-87).  mean/rstd: (rows) fp32, saved
- * for the backward pass (the reference recomputes them instead). */
-int tf_layernorm_fwd(void* stream, int dtype, int64_t rows, int64_t d,
+ * for the backward pass (the reference recomputes them instead).
+ * gamma, beta (and dgamma, dbeta below) have `param_dtype`: `dtype`, or TF_F32
+ * for fp32 master parameters used as they are. */
+int tf_layernorm_fwd(void* stream, int dtype, int param_dtype, int64_t rows, int64_t d,
                      const void* x, int64_t ldx, const void* gamma, const void* beta,
                      float eps, void* y, int64_t ldy, float* mean, float* rstd);
 
@@ -135,7 +137,7 @@ int tf_layernorm_fwd(void* stream, int dtype, int64_t rows, int64_t d,
  * reduction.  Replaces dx_layernorm (kernels/layernorm.py:140-162) and
  * layernorm_da_db (kernels/layernorm.py:226-259, with its reductions.py
  * second stage).  partial: fp32 scratch of tf_layernorm_bwd_partial_bytes(). */
-int tf_layernorm_bwd(void* stream, int dtype, int64_t rows, int64_t d,
+int tf_layernorm_bwd(void* stream, int dtype, int param_dtype, int64_t rows, int64_t d,
                      const void* dy, int64_t lddy, const void* x, int64_t ldx,
                      const void* gamma, const float* mean, const float* rstd,
                      void* dx, int64_t lddx, void* dgamma, void* dbeta,

@@ -88,9 +88,10 @@ def test_attention_rejects_bad_shapes():
 
 def test_row_kernels_reject_bad_arguments():
     lib = _lib.load()
-    assert lib.tf_layernorm_fwd(None, 2, 4, 64, FAKE, 64, FAKE, FAKE, 1e-5, FAKE, 64, FAKE, FAKE) == -2
-    assert lib.tf_layernorm_fwd(None, 0, 4, 64, FAKE, 32, FAKE, FAKE, 1e-5, FAKE, 64, FAKE, FAKE) == -1
-    assert lib.tf_layernorm_bwd(None, 0, 4, 64, FAKE, 64, FAKE, 64, FAKE, FAKE, FAKE, FAKE, 64, FAKE, FAKE,
+    assert lib.tf_layernorm_fwd(None, 2, 2, 4, 64, FAKE, 64, FAKE, FAKE, 1e-5, FAKE, 64, FAKE, FAKE) == -2
+    assert lib.tf_layernorm_fwd(None, 0, 1, 4, 64, FAKE, 64, FAKE, FAKE, 1e-5, FAKE, 64, FAKE, FAKE) == -2   # bf16 params, fp16 x
+    assert lib.tf_layernorm_fwd(None, 0, 0, 4, 64, FAKE, 32, FAKE, FAKE, 1e-5, FAKE, 64, FAKE, FAKE) == -1
+    assert lib.tf_layernorm_bwd(None, 0, 0, 4, 64, FAKE, 64, FAKE, 64, FAKE, FAKE, FAKE, FAKE, 64, FAKE, FAKE,
                                 None, 0) == -5
     assert lib.tf_layernorm_bwd_partial_bytes(8192, 1024) == 512 * 2 * 1024 * 4
     assert lib.tf_softmax_fwd(None, 0, 4, 0, FAKE, 64, FAKE, 64) == -1

@@ -75,6 +75,24 @@ def test_layernorm_headline_shape_and_autocast(dev):
     assert_close(x.grad, dx, name="dx", atol=2e-2)
 
 
+def test_layernorm_fp32_parameters_direct(dev):
+    """fp32 gamma / beta with 16-bit activations (master parameters under autocast) are
+    read by the kernel as they are; their gradients come back in fp32."""
+    g = torch.Generator().manual_seed(5)
+    x = (1.0 + torch.randn(2, 70, 333, generator=g)).half()
+    gamma, beta = torch.randn(333, generator=g), torch.randn(333, generator=g)
+    dy = torch.randn(2, 70, 333, generator=g).half()
+    xd = x.to(dev).requires_grad_(True)
+    gd, bd = gamma.to(dev).requires_grad_(True), beta.to(dev).requires_grad_(True)
+    y = T.layer_norm.apply(xd, gd, bd, 1e-5)
+    y.backward(dy.to(dev))
+    assert y.dtype == torch.float16 and gd.grad.dtype == torch.float32
+    assert_close(y, R.layer_norm(x, gamma, beta), name="y")
+    dx, dg, db = R.layer_norm_bwd(x, gamma, dy)
+    assert_close(xd.grad, dx, name="dx", atol=2e-2)
+    assert rel_l2(gd.grad, dg) < 1e-3 and rel_l2(bd.grad, db) < 1e-3
+
+
 def test_layernorm_rejects_fp32_and_2d(dev):
     with pytest.raises(TypeError):   # reference kernels/layernorm.py:71 asserts fp16
         T.layer_norm.apply(torch.zeros(1, 4, 8, device=dev), torch.ones(8, device=dev), torch.zeros(8, device=dev), 1e-5)

@@ -22,7 +22,12 @@ def _cast(value, dtype):
     return value
 
 
-def amp_fwd(fwd):
+def amp_fwd(fwd=None, *, keep=()):
+    """``keep``: positions of arguments that are passed through uncast (small fp32
+    parameter vectors the kernel reads directly)."""
+    if fwd is None:
+        return functools.partial(amp_fwd, keep=keep)
+
     @functools.wraps(fwd)
     def wrapper(ctx, *args):
         ctx._dtype = torch.get_autocast_dtype("cuda")
@@ -32,7 +37,8 @@ def amp_fwd(fwd):
         if torch.is_autocast_enabled("cuda"):
             dtype = torch.bfloat16 if ctx._dtype == torch.bfloat16 else torch.float16
             with torch.autocast(device_type="cuda", enabled=False):
-                return fwd(ctx, *_cast(args, dtype))
+                cast = tuple(a if i in keep else _cast(a, dtype) for i, a in enumerate(args))
+                return fwd(ctx, *cast)
         return fwd(ctx, *args)
 
     return wrapper

@@ -8,12 +8,23 @@ namespace tfa {
 
 constexpr int kRowsPerBlock = 4;  // 4 waves per workgroup, one row each
 
+// 8 consecutive affine parameters as fp32; TP = the 16-bit activation type or float
+// (fp32 master parameters are read as they are, no 16-bit copy is made first).
+template <typename TP> __device__ __forceinline__ void load8(const TP* p, float (&v)[8]) { Chunk<TP>::load(p, v); }
+template <> __device__ __forceinline__ void load8<float>(const float* p, float (&v)[8]) {
+  float a[4], b[4];
+  Chunk<float>::load(p, a);
+  Chunk<float>::load(p + 4, b);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { v[i] = a[i]; v[4 + i] = b[i]; }
+}
+
 // ---------------------------------------------------------------------------
 // LayerNorm forward.  NV = 16-byte chunks per lane (row length <= NV*64*8).
 // ---------------------------------------------------------------------------
-template <typename T, int NV>
+template <typename T, typename TP, int NV>
 __global__ __launch_bounds__(256) void ln_fwd_vec(int64_t rows, int d, const T* __restrict__ x, int64_t ldx,
-                                                   const T* __restrict__ gamma, const T* __restrict__ beta,
+                                                   const TP* __restrict__ gamma, const TP* __restrict__ beta,
                                                    float eps, T* __restrict__ y, int64_t ldy,
                                                    float* __restrict__ mean_out, float* __restrict__ rstd_out) {
   const int lane = threadIdx.x & 63;
@@ -53,8 +64,8 @@ __global__ __launch_bounds__(256) void ln_fwd_vec(int64_t rows, int d, const T* 
     const int c = lane + i * 64;
     if (c < nchunk) {
       float g[8], b[8], o[8];
-      Chunk<T>::load(gamma + c * 8, g);
-      Chunk<T>::load(beta + c * 8, b);
+      load8<TP>(gamma + c * 8, g);
+      load8<TP>(beta + c * 8, b);
 #pragma unroll
       for (int e = 0; e < 8; ++e) o[e] = (v[i][e] - mean) * rstd * g[e] + b[e];
       Chunk<T>::store(yr + c * 8, o);
@@ -64,9 +75,9 @@ __global__ __launch_bounds__(256) void ln_fwd_vec(int64_t rows, int d, const T* 
 
 // Any row length / alignment: scalar loads, three passes over the row (the
 // second and third come from cache).
-template <typename T>
+template <typename T, typename TP>
 __global__ __launch_bounds__(256) void ln_fwd_any(int64_t rows, int d, const T* __restrict__ x, int64_t ldx,
-                                                   const T* __restrict__ gamma, const T* __restrict__ beta,
+                                                   const TP* __restrict__ gamma, const TP* __restrict__ beta,
                                                    float eps, T* __restrict__ y, int64_t ldy,
                                                    float* __restrict__ mean_out, float* __restrict__ rstd_out) {
   const int lane = threadIdx.x & 63;
@@ -90,10 +101,10 @@ __global__ __launch_bounds__(256) void ln_fwd_any(int64_t rows, int d, const T* 
 // dx is written per row; dgamma/dbeta partial sums stay in registers, are
 // summed over the 4 waves through LDS and land in partial[b][0|1][d].
 // ---------------------------------------------------------------------------
-template <typename T, int NV>
+template <typename T, typename TP, int NV>
 __global__ __launch_bounds__(256) void ln_bwd_vec(int64_t rows, int d, const T* __restrict__ dy, int64_t lddy,
                                                    const T* __restrict__ x, int64_t ldx,
-                                                   const T* __restrict__ gamma, const float* __restrict__ mean,
+                                                   const TP* __restrict__ gamma, const float* __restrict__ mean,
                                                    const float* __restrict__ rstd, T* __restrict__ dx,
                                                    int64_t lddx, float* __restrict__ partial) {
   extern __shared__ float red[];  // [4][d]
@@ -106,7 +117,7 @@ __global__ __launch_bounds__(256) void ln_bwd_vec(int64_t rows, int d, const T* 
     const int c = lane + i * 64;
 #pragma unroll
     for (int e = 0; e < 8; ++e) { dg[i][e] = 0.f; db[i][e] = 0.f; g[i][e] = 0.f; }
-    if (c < nchunk) Chunk<T>::load(gamma + c * 8, g[i]);
+    if (c < nchunk) load8<TP>(gamma + c * 8, g[i]);
   }
   const float inv_d = 1.0f / (float)d;
   for (int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + wave; row < rows;
@@ -170,10 +181,10 @@ __global__ __launch_bounds__(256) void ln_bwd_vec(int64_t rows, int d, const T* 
   }
 }
 
-template <typename T>
+template <typename T, typename TP>
 __global__ __launch_bounds__(256) void ln_bwd_any(int64_t rows, int d, const T* __restrict__ dy, int64_t lddy,
                                                    const T* __restrict__ x, int64_t ldx,
-                                                   const T* __restrict__ gamma, const float* __restrict__ mean,
+                                                   const TP* __restrict__ gamma, const float* __restrict__ mean,
                                                    const float* __restrict__ rstd, T* __restrict__ dx,
                                                    int64_t lddx, float* __restrict__ partial) {
   // One workgroup per slice of rows; every thread owns columns tid, tid+256, ...
@@ -355,7 +366,7 @@ static int pick_nv(int64_t nchunk) {
   return 0;
 }
 
-template <typename T>
+template <typename T, typename TP>
 static int ln_fwd_launch(hipStream_t st, int64_t rows, int64_t d, const void* x, int64_t ldx, const void* gamma,
                          const void* beta, float eps, void* y, int64_t ldy, float* mean, float* rstd) {
   const dim3 grid((unsigned)ceil_div(rows, kRowsPerBlock)), block(256);
@@ -363,7 +374,7 @@ static int ln_fwd_launch(hipStream_t st, int64_t rows, int64_t d, const void* x,
                    aligned16(beta);
   const int nv = vec ? pick_nv(d / 8) : 0;
 #define LN_FWD(NV)                                                                                           \
-  ln_fwd_vec<T, NV><<<grid, block, 0, st>>>(rows, (int)d, (const T*)x, ldx, (const T*)gamma, (const T*)beta, \
+  ln_fwd_vec<T, TP, NV><<<grid, block, 0, st>>>(rows, (int)d, (const T*)x, ldx, (const TP*)gamma, (const TP*)beta, \
                                             eps, (T*)y, ldy, mean, rstd)
   switch (nv) {
     case 1: LN_FWD(1); break;
@@ -371,7 +382,7 @@ static int ln_fwd_launch(hipStream_t st, int64_t rows, int64_t d, const void* x,
     case 4: LN_FWD(4); break;
     case 8: LN_FWD(8); break;
     default:
-      ln_fwd_any<T><<<grid, block, 0, st>>>(rows, (int)d, (const T*)x, ldx, (const T*)gamma, (const T*)beta, eps,
+      ln_fwd_any<T, TP><<<grid, block, 0, st>>>(rows, (int)d, (const T*)x, ldx, (const TP*)gamma, (const TP*)beta, eps,
                                             (T*)y, ldy, mean, rstd);
   }
 #undef LN_FWD
@@ -384,7 +395,7 @@ static int ln_bwd_parts(int64_t rows) {
   return (int)(g < 512 ? g : 512);
 }
 
-template <typename T>
+template <typename T, typename TP>
 static int ln_bwd_launch(hipStream_t st, int64_t rows, int64_t d, const void* dy, int64_t lddy, const void* x,
                          int64_t ldx, const void* gamma, const float* mean, const float* rstd, void* dx,
                          int64_t lddx, void* dgamma, void* dbeta, float* partial) {
@@ -394,20 +405,20 @@ static int ln_bwd_launch(hipStream_t st, int64_t rows, int64_t d, const void* dy
   const int nv = vec ? pick_nv(d / 8) : 0;
   const size_t lds = (size_t)4 * d * sizeof(float);
 #define LN_BWD(NV)                                                                                          \
-  ln_bwd_vec<T, NV><<<dim3(parts), dim3(256), lds, st>>>(rows, (int)d, (const T*)dy, lddy, (const T*)x, ldx, \
-                                                         (const T*)gamma, mean, rstd, (T*)dx, lddx, partial)
+  ln_bwd_vec<T, TP, NV><<<dim3(parts), dim3(256), lds, st>>>(rows, (int)d, (const T*)dy, lddy, (const T*)x, ldx, \
+                                                             (const TP*)gamma, mean, rstd, (T*)dx, lddx, partial)
   switch (nv) {
     case 1: LN_BWD(1); break;
     case 2: LN_BWD(2); break;
     case 4: LN_BWD(4); break;
     case 8: LN_BWD(8); break;
     default:
-      ln_bwd_any<T><<<dim3(parts), dim3(256), 0, st>>>(rows, (int)d, (const T*)dy, lddy, (const T*)x, ldx,
-                                                       (const T*)gamma, mean, rstd, (T*)dx, lddx, partial);
+      ln_bwd_any<T, TP><<<dim3(parts), dim3(256), 0, st>>>(rows, (int)d, (const T*)dy, lddy, (const T*)x, ldx,
+                                                           (const TP*)gamma, mean, rstd, (T*)dx, lddx, partial);
   }
 #undef LN_BWD
   TF_CHECK_LAUNCH();
-  ln_bwd_reduce<T><<<dim3(ceil_div(2 * d, 16)), dim3(256), 0, st>>>(parts, (int)d, partial, (T*)dgamma, (T*)dbeta);
+  ln_bwd_reduce<TP><<<dim3(ceil_div(2 * d, 16)), dim3(256), 0, st>>>(parts, (int)d, partial, (TP*)dgamma, (TP*)dbeta);
   TF_CHECK_LAUNCH();
   return TF_OK;
 }
@@ -461,15 +472,21 @@ static bool bad_rows(int64_t rows, int64_t n, int64_t ld) {
 
 using namespace tfa;
 
-extern "C" int tf_layernorm_fwd(void* stream, int dtype, int64_t rows, int64_t d, const void* x, int64_t ldx,
-                                const void* gamma, const void* beta, float eps, void* y, int64_t ldy,
+extern "C" int tf_layernorm_fwd(void* stream, int dtype, int param_dtype, int64_t rows, int64_t d, const void* x,
+                                int64_t ldx, const void* gamma, const void* beta, float eps, void* y, int64_t ldy,
                                 float* mean, float* rstd) {
   if (!x || !gamma || !beta || !y || !mean || !rstd) return TF_EINVAL;
   if (bad_rows(rows, d, ldx) || ldy < d) return TF_EINVAL;
   if (rows == 0) return TF_OK;
   hipStream_t st = (hipStream_t)stream;
-  if (dtype == TF_F16) return ln_fwd_launch<f16>(st, rows, d, x, ldx, gamma, beta, eps, y, ldy, mean, rstd);
-  if (dtype == TF_BF16) return ln_fwd_launch<bf16>(st, rows, d, x, ldx, gamma, beta, eps, y, ldy, mean, rstd);
+  if (param_dtype != dtype && param_dtype != TF_F32) return TF_EDTYPE;
+  const bool pf = param_dtype == TF_F32;
+  if (dtype == TF_F16)
+    return pf ? ln_fwd_launch<f16, float>(st, rows, d, x, ldx, gamma, beta, eps, y, ldy, mean, rstd)
+              : ln_fwd_launch<f16, f16>(st, rows, d, x, ldx, gamma, beta, eps, y, ldy, mean, rstd);
+  if (dtype == TF_BF16)
+    return pf ? ln_fwd_launch<bf16, float>(st, rows, d, x, ldx, gamma, beta, eps, y, ldy, mean, rstd)
+              : ln_fwd_launch<bf16, bf16>(st, rows, d, x, ldx, gamma, beta, eps, y, ldy, mean, rstd);
   return TF_EDTYPE;
 }
 
@@ -478,7 +495,8 @@ extern "C" int64_t tf_layernorm_bwd_partial_bytes(int64_t rows, int64_t d) {
   return (int64_t)ln_bwd_parts(rows) * 2 * d * (int64_t)sizeof(float);
 }
 
-extern "C" int tf_layernorm_bwd(void* stream, int dtype, int64_t rows, int64_t d, const void* dy, int64_t lddy,
+extern "C" int tf_layernorm_bwd(void* stream, int dtype, int param_dtype, int64_t rows, int64_t d, const void* dy,
+                                int64_t lddy,
                                 const void* x, int64_t ldx, const void* gamma, const float* mean,
                                 const float* rstd, void* dx, int64_t lddx, void* dgamma, void* dbeta,
                                 float* partial, int64_t partial_bytes) {
@@ -486,10 +504,12 @@ extern "C" int tf_layernorm_bwd(void* stream, int dtype, int64_t rows, int64_t d
   if (bad_rows(rows, d, ldx) || lddy < d || lddx < d || rows == 0) return TF_EINVAL;
   if (!partial || partial_bytes < tf_layernorm_bwd_partial_bytes(rows, d)) return TF_EWORKSPACE;
   hipStream_t st = (hipStream_t)stream;
-  if (dtype == TF_F16)
-    return ln_bwd_launch<f16>(st, rows, d, dy, lddy, x, ldx, gamma, mean, rstd, dx, lddx, dgamma, dbeta, partial);
-  if (dtype == TF_BF16)
-    return ln_bwd_launch<bf16>(st, rows, d, dy, lddy, x, ldx, gamma, mean, rstd, dx, lddx, dgamma, dbeta, partial);
+  if (param_dtype != dtype && param_dtype != TF_F32) return TF_EDTYPE;
+#define LN_BWD_GO(T, TP) \
+  return ln_bwd_launch<T, TP>(st, rows, d, dy, lddy, x, ldx, gamma, mean, rstd, dx, lddx, dgamma, dbeta, partial)
+  if (dtype == TF_F16) { if (param_dtype == TF_F32) LN_BWD_GO(f16, float); else LN_BWD_GO(f16, f16); }
+  if (dtype == TF_BF16) { if (param_dtype == TF_F32) LN_BWD_GO(bf16, float); else LN_BWD_GO(bf16, bf16); }
+#undef LN_BWD_GO
   return TF_EDTYPE;
 }
 

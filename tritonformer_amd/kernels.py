@@ -237,13 +237,14 @@ def _check_ln(x, d):
 def layernorm_fwd(x, alpha, beta, eps):
     """-> (y, mean, rstd); reference kernels/layernorm.py:64-87."""
     _check_ln(x, alpha.shape[0])
-    if alpha.dtype != x.dtype or beta.dtype != x.dtype:
-        raise TypeError("LayerNorm parameters must have the input's dtype")
+    if alpha.dtype != beta.dtype or alpha.dtype not in (x.dtype, torch.float32):
+        raise TypeError("LayerNorm parameters must have the input's dtype or be float32")
+    require_cuda(alpha, beta)
     x2, rows, d = _rows2d(x)
     y = torch.empty(x.shape, dtype=x.dtype, device=x.device)
     mean = torch.empty((rows,), dtype=torch.float32, device=x.device)
     rstd = torch.empty((rows,), dtype=torch.float32, device=x.device)
-    check(load().tf_layernorm_fwd(stream_ptr(), dtype_code(x.dtype), rows, d, x2.data_ptr(), d,
+    check(load().tf_layernorm_fwd(stream_ptr(), dtype_code(x.dtype), dtype_code(alpha.dtype), rows, d, x2.data_ptr(), d,
                                   alpha.contiguous().data_ptr(), beta.contiguous().data_ptr(), float(eps),
                                   y.data_ptr(), d, mean.data_ptr(), rstd.data_ptr()))
     return y, mean, rstd
@@ -256,11 +257,12 @@ def layernorm_bwd(grad_out, x, alpha, mean, rstd):
     x2, rows, d = _rows2d(x)
     g2, _, _ = _rows2d(grad_out)
     dx = torch.empty(x.shape, dtype=x.dtype, device=x.device)
-    da = torch.empty((d,), dtype=x.dtype, device=x.device)
-    db = torch.empty((d,), dtype=x.dtype, device=x.device)
+    da = torch.empty((d,), dtype=alpha.dtype, device=x.device)
+    db = torch.empty((d,), dtype=alpha.dtype, device=x.device)
     pb = lib.tf_layernorm_bwd_partial_bytes(rows, d)
     part = torch.empty(pb, dtype=torch.uint8, device=x.device)
-    check(lib.tf_layernorm_bwd(stream_ptr(), dtype_code(x.dtype), rows, d, g2.data_ptr(), d, x2.data_ptr(), d,
+    check(lib.tf_layernorm_bwd(stream_ptr(), dtype_code(x.dtype), dtype_code(alpha.dtype), rows, d, g2.data_ptr(), d,
+                               x2.data_ptr(), d,
                                alpha.contiguous().data_ptr(), mean.data_ptr(), rstd.data_ptr(), dx.data_ptr(), d,
                                da.data_ptr(), db.data_ptr(), part.data_ptr(), pb))
     return dx, da, db

@@ -8,7 +8,7 @@ from .kernels import layernorm_bwd, layernorm_fwd
 
 class LayerNorm(Function):
     @staticmethod
-    @amp_fwd
+    @amp_fwd(keep=(1, 2))  # fp32 master gamma / beta are read by the kernel as they are
     def forward(ctx, input, alpha, beta, eps):
         x_ln, mean, rstd = layernorm_fwd(input, alpha, beta, eps)
         ctx.save_for_backward(input, alpha, mean, rstd)
