@@ -71,14 +71,20 @@ int tf_gemm(void* stream, int dtype, int layout_a, int layout_b,
             const void* A, int64_t lda, const void* B, int64_t ldb,
             void* C, int64_t ldc, const void* bias, int relu,
             void* workspace, int64_t workspace_bytes);
-/* As tf_gemm with C stored as `out_dtype`: either `dtype` or TF_F32 (fp32 weight
- * gradients for fp32 master weights, skipping the separate 16->32 bit cast pass
- * autograd would otherwise run; the reference keeps fp16 parameters and has no
- * such case). */
+/* As tf_gemm with two extras.
+ * `out_dtype`: C is stored as `dtype` or as TF_F32 (fp32 weight gradients for
+ * fp32 master weights, skipping the separate 16->32 bit cast pass autograd would
+ * otherwise run; the reference keeps fp16 parameters and has no such case).
+ * `mask_act` (NULL, or an (M, N) matrix of `dtype`, leading dimension ld_mask):
+ * C[m,n] is zeroed where mask_act[m,n] <= 0 -- the ReLU gradient mask of
+ * kernels/activation.py:27-44 applied while the input gradient of the following
+ * layer is written, instead of in a pass of its own; excludes bias and relu,
+ * and such a call never splits the contraction (no workspace needed). */
 int tf_gemm_out(void* stream, int dtype, int out_dtype, int layout_a, int layout_b,
                 int64_t M, int64_t N, int64_t K,
                 const void* A, int64_t lda, const void* B, int64_t ldb,
                 void* C, int64_t ldc, const void* bias, int relu,
+                const void* mask_act, int64_t ld_mask,
                 void* workspace, int64_t workspace_bytes);
 int64_t tf_gemm_workspace_bytes(int layout_a, int layout_b, int64_t M, int64_t N, int64_t K);
 /* Diagnostic, no counterpart in the reference (whose Triton autotuner picks

@@ -65,7 +65,10 @@ def test_gemm_rejects_bad_arguments():
     assert need > 0 and need % (1024 * 1024 * 4) == 0
     assert g(None, 0, 1, 1, 1024, 1024, 8192, FAKE, 1024, FAKE, 1024, FAKE, 1024, None, 0, None, 0) == -5
     assert lib.tf_gemm_workspace_bytes(0, 1, 8192, 4096, 1024) == 0
-    assert lib.tf_gemm_out(None, 0, 1, 0, 1, 64, 64, 64, *ok_tail) == -2                        # bf16 out of fp16 in
+    out_tail = (FAKE, 64, FAKE, 64, FAKE, 64, None, 0, None, 0, None, 0)
+    assert lib.tf_gemm_out(None, 0, 1, 0, 1, 64, 64, 64, *out_tail) == -2                       # bf16 out of fp16 in
+    assert lib.tf_gemm_out(None, 0, 0, 0, 1, 64, 64, 64, FAKE, 64, FAKE, 64, FAKE, 64, None, 1, FAKE, 64,
+                           None, 0) == -1                                                        # mask with ReLU
 
 
 def test_attention_rejects_bad_shapes():

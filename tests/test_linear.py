@@ -177,3 +177,38 @@ def test_logits_projection_shape(dev):
     dx, dw, _ = R.linear_bwd(x.detach(), w.detach(), dy)
     assert_close(x.grad, dx, name="dx", atol=2e-2)
     assert rel_l2(w.grad, dw) < 1e-3
+
+
+@pytest.mark.parametrize("dims,use_bias", [((2, 128, 256, 1024), False), ((3, 77, 136, 264), True),
+                                           ((1, 100, 333, 129), True)])
+def test_fused_mlp_equals_two_functions(dims, use_bias, dev):
+    """mlp_fused_relu must equal linear_fused_(bias_)relu followed by linear_(no_)bias bit for
+    bit (same GEMM calls; the mask is applied in the write-out instead of a separate pass)."""
+    b, m, d, f = dims
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(b, m, d, generator=g).half().to(dev)
+    w1 = (torch.randn(d, f, generator=g) / d ** 0.5).half().to(dev)
+    w2 = (torch.randn(f, d, generator=g) / f ** 0.5).half().to(dev)
+    b1 = torch.randn(f, generator=g).half().to(dev) if use_bias else None
+    b2 = torch.randn(d, generator=g).half().to(dev) if use_bias else None
+    dy = torch.randn(b, m, d, generator=g).half().to(dev)
+
+    def leaves():
+        return [t.clone().requires_grad_(True) if t is not None else None for t in (x, w1, b1, w2, b2)]
+
+    a = leaves()
+    ya = T.mlp_fused_relu.apply(*a)
+    ya.backward(dy)
+    c = leaves()
+    if use_bias:
+        yb = T.linear_bias.apply(T.linear_fused_bias_relu.apply(c[0], c[1], c[2]), c[3], c[4])
+    else:
+        yb = T.linear_no_bias.apply(T.linear_fused_relu.apply(c[0], c[1]), c[3])
+    yb.backward(dy)
+    assert torch.equal(ya, yb)
+    for ta, tb in zip(a, c):
+        if ta is not None:
+            assert torch.equal(ta.grad, tb.grad)
+    y_ref = R.linear(R.linear(x.cpu(), w1.cpu(), b1.cpu() if use_bias else None, True).half(), w2.cpu(),
+                     b2.cpu() if use_bias else None)
+    assert_close(ya, y_ref, name="mlp y", atol=2e-2)

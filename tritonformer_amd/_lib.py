@@ -22,7 +22,8 @@ SIGNATURES = {
     "tf_status_string": (_c.c_char_p, [_i]),
     "tf_version": (_i, []),
     "tf_gemm": (_i, [_vp, _i, _i, _i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i, _vp, _i64]),
-    "tf_gemm_out": (_i, [_vp, _i, _i, _i, _i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i, _vp, _i64]),
+    "tf_gemm_out": (_i, [_vp, _i, _i, _i, _i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i, _vp, _i64,
+                         _vp, _i64]),
     "tf_gemm_workspace_bytes": (_i64, [_i, _i, _i64, _i64, _i64]),
     "tf_gemm_tune": (_i, [_i, _i]),
     "tf_gemm_debug_flags": (_i, [_i]),

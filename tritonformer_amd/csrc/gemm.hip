@@ -42,6 +42,8 @@ struct GemmParams {
   int tiles_m, tiles_n;
   int flags;  // bit 0: skip the XCD remap (diagnostic)
   int out_f32;  // C holds fp32 instead of T
+  const void* mask;  // optional (M, N) activation of type T: C = mask > 0 ? C : 0
+  int64_t ldmask;
 };
 
 // ---------------------------------------------------------------------------
@@ -156,6 +158,12 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
               if (n + e < p.N) dst[e] = v[e];
           }
         } else {
+          if (p.mask) {
+            const T* mk = (const T*)p.mask + (int64_t)m * p.ldmask + n;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (n + e < p.N && !((float)mk[e] > 0.f)) v[e] = 0.f;  // no bias / ReLU with a mask (host check)
+          }
           if (p.out_f32) {
             float* Cf = reinterpret_cast<float*>(p.C) + (int64_t)m * p.ldc + n;
 #pragma unroll
@@ -437,9 +445,29 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x16 (&
 #pragma unroll
     for (int rr = 0; rr < 32 / RPI; ++rr) {
       const int r = rr * RPI + lane / CH, c = lane % CH;
-      const u32x4 val = lds_ld16(mine, r * ROWB + c * 16);
+      u32x4 val = lds_ld16(mine, r * ROWB + c * 16);
       const int m = m0 + wm * WTM + i * 32 + r, n = nbase + c * EPC;
-      if (m < p.M && n < p.N) st16(C + (int64_t)m * p.ldc + n, val);
+      if (m < p.M && n < p.N) {
+        if (p.mask) {  // ReLU gradient mask fused into the write-out: zero where the activation is not positive
+          const T* mk = (const T*)p.mask + (int64_t)m * p.ldmask + n;
+          if constexpr (ES == 2) {
+            const typename Vec<T>::v8 mv = __builtin_bit_cast(typename Vec<T>::v8, ld16(mk));
+            typename Vec<T>::v8 cv = __builtin_bit_cast(typename Vec<T>::v8, val);
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              if (!((float)mv[e] > 0.f)) cv[e] = (T)0.f;
+            val = __builtin_bit_cast(u32x4, cv);
+          } else {
+            const typename Vec<T>::v4 mv = *reinterpret_cast<const typename Vec<T>::v4*>(mk);
+            f32x4 cv = __builtin_bit_cast(f32x4, val);
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (!((float)mv[e] > 0.f)) cv[e] = 0.f;
+            val = __builtin_bit_cast(u32x4, cv);
+          }
+        }
+        st16(C + (int64_t)m * p.ldc + n, val);
+      }
     }
   }
 }
@@ -652,7 +680,7 @@ static int g_flags = env_int("TF_GEMM_FLAGS", 0);
 // rocprofv3 kernel durations on MI355X: one "round" of workgroups (one per CU)
 // costs a fixed part (launch, cold first loads, result write-out) plus a part
 // per 64-wide contraction step.
-static GemmPlan plan_for(int cfg, int64_t M, int64_t N, int64_t K, double* cost_us) {
+static GemmPlan plan_for(int cfg, int64_t M, int64_t N, int64_t K, double* cost_us, bool allow_split) {
   GemmPlan pl;
   pl.cfg = cfg;
   pl.bm = kCfgs[cfg].bm;
@@ -676,6 +704,7 @@ static GemmPlan plan_for(int cfg, int64_t M, int64_t N, int64_t K, double* cost_
     if (splits > 16) splits = 16;
   }
   if (g_force_splits > 0) splits = g_force_splits;
+  if (!allow_split) splits = 1;
   if (splits > ksteps) splits = ksteps > 0 ? ksteps : 1;
   const int64_t steps_per = (ksteps + splits - 1) / splits;
   pl.k_per_split = (int)(steps_per * pl.bk);
@@ -692,12 +721,12 @@ static GemmPlan plan_for(int cfg, int64_t M, int64_t N, int64_t K, double* cost_
   return pl;
 }
 
-static GemmPlan make_plan(int64_t M, int64_t N, int64_t K, bool vec) {
+static GemmPlan make_plan(int64_t M, int64_t N, int64_t K, bool vec, bool allow_split = true) {
   const bool dma = vec && K % 64 == 0;
   if (g_force_cfg >= 0 && g_force_cfg < kNumCfgs) {
     int cfg = g_force_cfg;
     if (kCfgs[cfg].dma && !dma) cfg = kCfgs[cfg].bm * kCfgs[cfg].bn >= 256 * 256 ? 0 : 1;  // register-staged twin
-    return plan_for(cfg, M, N, K, nullptr);
+    return plan_for(cfg, M, N, K, nullptr, allow_split);
   }
   // candidates: 256x256 and 256x128 / 128x128 tiles, direct-to-LDS kernels when their
   // preconditions hold, the register-staged twins otherwise
@@ -705,11 +734,11 @@ static GemmPlan make_plan(int64_t M, int64_t N, int64_t K, bool vec) {
   const int cand_reg[2] = {0, 1};
   const int* cand = dma ? cand_dma : cand_reg;
   const int ncand = dma ? 3 : 2;
-  GemmPlan best = plan_for(cand[0], M, N, K, nullptr);
+  GemmPlan best = plan_for(cand[0], M, N, K, nullptr, allow_split);
   double best_cost = 1e30;
   for (int i = 0; i < ncand; ++i) {
     double c;
-    const GemmPlan pl = plan_for(cand[i], M, N, K, &c);
+    const GemmPlan pl = plan_for(cand[i], M, N, K, &c, allow_split);
     if (c < best_cost) { best_cost = c; best = pl; }
   }
   return best;
@@ -831,14 +860,16 @@ extern "C" int64_t tf_gemm_workspace_bytes(int layout_a, int layout_b, int64_t M
 extern "C" int tf_gemm(void* stream, int dtype, int layout_a, int layout_b, int64_t M, int64_t N, int64_t K,
                        const void* A, int64_t lda, const void* B, int64_t ldb, void* C, int64_t ldc,
                        const void* bias, int relu, void* workspace, int64_t workspace_bytes) {
-  return tf_gemm_out(stream, dtype, dtype, layout_a, layout_b, M, N, K, A, lda, B, ldb, C, ldc, bias, relu, workspace,
-                     workspace_bytes);
+  return tf_gemm_out(stream, dtype, dtype, layout_a, layout_b, M, N, K, A, lda, B, ldb, C, ldc, bias, relu, nullptr, 0,
+                     workspace, workspace_bytes);
 }
 
 extern "C" int tf_gemm_out(void* stream, int dtype, int out_dtype, int layout_a, int layout_b, int64_t M, int64_t N,
                            int64_t K, const void* A, int64_t lda, const void* B, int64_t ldb, void* C, int64_t ldc,
-                           const void* bias, int relu, void* workspace, int64_t workspace_bytes) {
+                           const void* bias, int relu, const void* mask_act, int64_t ld_mask, void* workspace,
+                           int64_t workspace_bytes) {
   if (!A || !B || !C) return TF_EINVAL;
+  if (mask_act && (bias || relu || ld_mask < N)) return TF_EINVAL;
   if (out_dtype != dtype && out_dtype != TF_F32) return TF_EDTYPE;
   if (M <= 0 || N <= 0 || K <= 0 || M > 0x7fffff00 || N > 0x7fffff00 || K > 0x7fffff00) return TF_EINVAL;
   if ((layout_a != TF_OP_KMAJOR && layout_a != TF_OP_KMINOR) || (layout_b != TF_OP_KMAJOR && layout_b != TF_OP_KMINOR))
@@ -852,8 +883,9 @@ extern "C" int tf_gemm_out(void* stream, int dtype, int out_dtype, int layout_a,
     return TF_EALIGN;
 
   const bool vec = aligned16(A) && aligned16(B) && aligned16(C) && (!bias || aligned16(bias)) && a_contig % 8 == 0 &&
-                   b_contig % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 && N % 8 == 0 && ldc % 8 == 0;
-  const GemmPlan pl = make_plan(M, N, K, vec);
+                   b_contig % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 && N % 8 == 0 && ldc % 8 == 0 &&
+                   (!mask_act || (aligned16(mask_act) && ld_mask % 8 == 0));
+  const GemmPlan pl = make_plan(M, N, K, vec, mask_act == nullptr);
   const int64_t need = pl.splits > 1 ? (int64_t)pl.splits * M * N * (int64_t)sizeof(float) : 0;
   if (need > 0 && (!workspace || workspace_bytes < need)) return TF_EWORKSPACE;
   if (need > 0 && !aligned16(workspace)) return TF_EALIGN;
@@ -868,6 +900,8 @@ extern "C" int tf_gemm_out(void* stream, int dtype, int out_dtype, int layout_a,
   p.tiles_m = pl.tiles_m; p.tiles_n = pl.tiles_n;
   p.flags = g_flags;
   p.out_f32 = out_dtype == TF_F32 ? 1 : 0;
+  p.mask = mask_act;
+  p.ldmask = ld_mask;
   hipStream_t st = (hipStream_t)stream;
   if (dtype == TF_F16) return gemm_dispatch<f16>(st, layout_a, layout_b, vec, pl, p);
   return gemm_dispatch<bf16>(st, layout_a, layout_b, vec, pl, p);

@@ -28,13 +28,14 @@ def _gemm_ws(la, lb, m, n, k):
     return load().tf_gemm_workspace_bytes(la, lb, m, n, k)
 
 
-def _gemm(dtype, la, lb, m, n, k, a, lda, b, ldb, c, ldc, bias, relu):
+def _gemm(dtype, la, lb, m, n, k, a, lda, b, ldb, c, ldc, bias, relu, mask=None):
     lib = load()
-    ws_bytes = _gemm_ws(la, lb, m, n, k)
+    ws_bytes = 0 if mask is not None else _gemm_ws(la, lb, m, n, k)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=c.device) if ws_bytes else None
     check(lib.tf_gemm_out(stream_ptr(), dtype_code(dtype), dtype_code(c.dtype), la, lb, m, n, k, a.data_ptr(), lda,
                           b.data_ptr(), ldb, c.data_ptr(), ldc, bias.data_ptr() if bias is not None else None,
-                          int(relu), ws.data_ptr() if ws is not None else None, ws_bytes))
+                          int(relu), mask.data_ptr() if mask is not None else None, n if mask is not None else 0,
+                          ws.data_ptr() if ws is not None else None, ws_bytes))
 
 
 def _check_linear(a, b, bias=None):
@@ -52,10 +53,20 @@ def _check_linear(a, b, bias=None):
     require_cuda(a, b, bias)
 
 
-def gemm(a, b, bias=None, fuse_relu=False):
+def gemm(a, b, bias=None, fuse_relu=False, mask_act=None):
     """``relu?(a @ b + bias)`` for a (B, S, in), b (in, out) — reference ``mm``
-    (kernels/gemm.py:361-401) and ``gemm`` (kernels/gemm.py:572-616)."""
+    (kernels/gemm.py:361-401) and ``gemm`` (kernels/gemm.py:572-616).
+    ``mask_act`` (same shape as the result): zero the result where it is <= 0,
+    i.e. reference ``mask_grad`` (kernels/activation.py:27-44) fused into the GEMM
+    that produces the gradient being masked."""
     _check_linear(a, b, bias)
+    if mask_act is not None:
+        if bias is not None or fuse_relu:
+            raise ValueError("mask_act excludes bias and ReLU")
+        if mask_act.shape != a.shape[:-1] + (b.shape[1],) or mask_act.dtype != a.dtype:
+            raise ValueError("mask_act must have the shape and dtype of the result")
+        if not mask_act.is_contiguous():
+            mask_act = mask_act.contiguous()
     a2, m, k = _rows2d(a)
     n = b.shape[1]
     if b.stride(-1) == 1 and b.stride(0) >= n:
@@ -68,12 +79,12 @@ def gemm(a, b, bias=None, fuse_relu=False):
     if bias is not None and not bias.is_contiguous():
         bias = bias.contiguous()
     out = torch.empty(a.shape[:-1] + (n,), dtype=a.dtype, device=a.device)
-    _gemm(a.dtype, KMAJOR, lb, m, n, k, a2, k, b, ldb, out, n, bias, fuse_relu)
+    _gemm(a.dtype, KMAJOR, lb, m, n, k, a2, k, b, ldb, out, n, bias, fuse_relu, mask_act)
     return out
 
 
-def mm(a, b, fuse_relu=False):
-    return gemm(a, b, None, fuse_relu)
+def mm(a, b, fuse_relu=False, mask_act=None):
+    return gemm(a, b, None, fuse_relu, mask_act)
 
 
 def mm_dw(x, grad, out_dtype=None):

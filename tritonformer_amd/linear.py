@@ -91,3 +91,35 @@ class LinearBiasReLU(Function):
         grad_input, grad_weights = _grads(ctx, grad_output, inputs, weights)
         grad_bias = unbroadcast_leading(grad_output) if ctx.needs_input_grad[2] else None
         return grad_input, grad_weights, grad_bias
+
+
+class MLPReLU(Function):
+    """Two linears with a ReLU between them as ONE autograd node:
+    ``apply(x, W1, b1_or_None, W2, b2_or_None) = relu(x W1 + b1) W2 + b2``.
+    Forward and weight/input gradients are the same GEMM calls as
+    LinearNoBiasReLU / LinearBiasReLU followed by LinearNoBias / LinearBias; being
+    one node lets the ReLU gradient mask ride on the write-out of dH = dY W2^T
+    instead of a pass of its own over (B, S, ffn).  No counterpart in the reference
+    (two Functions and an in-place mask kernel, linear.py:47-102)."""
+
+    @staticmethod
+    @amp_fwd
+    def forward(ctx, input, w1, b1, w2, b2):
+        hidden = gemm(input, w1, b1, True)
+        out = gemm(hidden, w2, b2, False)
+        ctx.save_for_backward(input, w1, w2, hidden)
+        ctx.has_bias = (b1 is not None, b2 is not None)
+        return out
+
+    @staticmethod
+    @amp_bwd
+    def backward(ctx, grad_output):
+        input, w1, w2, hidden = ctx.saved_tensors
+        f32 = torch.float32
+        grad_hidden = mm(grad_output, w2.T, mask_act=hidden)      # (dY W2^T) * (hidden > 0)
+        grad_w2 = mm_dw(hidden, grad_output, out_dtype=f32 if ctx.arg_dtypes[3] == f32 else None)
+        grad_b2 = unbroadcast_leading(grad_output) if ctx.has_bias[1] else None
+        grad_input = mm(grad_hidden, w1.T) if ctx.needs_input_grad[0] else None
+        grad_w1 = mm_dw(input, grad_hidden, out_dtype=f32 if ctx.arg_dtypes[1] == f32 else None)
+        grad_b1 = unbroadcast_leading(grad_hidden) if ctx.has_bias[0] else None
+        return grad_input, grad_w1, grad_b1, grad_w2, grad_b2

@@ -23,6 +23,7 @@ from . import (
     fast_causal_attention_qkvpacked,
     fast_causal_attention_with_bias,
     linear_no_bias,
+    mlp_fused_relu,
     shifted_cross_entropy_loss,
 )
 from . import nn as tnn
@@ -71,6 +72,9 @@ def generate_alibi_mask(seq_len: int, num_heads: int, device=None, dtype=torch.f
 # arithmetic per output element); False: three projections exactly as the reference
 # module does (transformer.py:158-182).
 FUSE_QKV = True
+# True: the MLP block is one autograd node (ReLU gradient mask fused into a GEMM write-out);
+# False: two Linear modules as in the reference (transformer.py:214-217).
+FUSE_MLP = True
 
 
 def _weights_init(model: nn.Module, num_layers: int) -> None:
@@ -146,6 +150,9 @@ class MLPBlock(nn.Module):
                                         bias=config.use_linear_bias)
 
     def forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
+        if FUSE_MLP:
+            return mlp_fused_relu.apply(hidden_states, self.dense_h_to_4h.weight, self.dense_h_to_4h.bias,
+                                        self.dense_4h_to_h.weight, self.dense_4h_to_h.bias)
         return self.dense_4h_to_h(self.dense_h_to_4h(hidden_states))
 
 
