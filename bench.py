@@ -154,7 +154,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-roofline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run one plain 1 GiB device-to-device copy kernel (known traffic: 1 GiB read, "
+                    help="also run one plain 1 GiB streaming kernel, dst = src + 1 (known traffic: 1 GiB read, "
                          "1 GiB written) so that rocprofv3 FETCH_SIZE / WRITE_SIZE readings can be scaled")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -226,7 +226,7 @@ def main():
     if args.calibrate_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device=device).normal_()
         dst = torch.empty_like(src)
-        dst.copy_(src)
+        torch.add(src, 1.0, out=dst)  # one elementwise kernel: reads 1 GiB, writes 1 GiB
         torch.cuda.synchronize()
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.workload)

@@ -150,6 +150,26 @@ int tf_layernorm_bwd(void* stream, int dtype, int param_dtype, int64_t rows, int
                      float* partial, int64_t partial_bytes);
 int64_t tf_layernorm_bwd_partial_bytes(int64_t rows, int64_t d);
 
+/* Residual addition fused into the LayerNorm that follows it:
+ *   sum = x + res (rounded to `dtype`, written out),  y = layernorm(sum).
+ * One kernel for the reference model's `hidden_states = residual + hidden_states`
+ * followed by the next LayerNorm (transformer.py:245-249, and :250 with the next
+ * layer's :243 or the final LayerNorm at :327); the results equal
+ * an elementwise addition followed by tf_layernorm_fwd bit for bit.
+ * The backward adds dsum, the gradient reaching `sum` along the residual
+ * stream, to the LayerNorm's own dx in fp32 before rounding: dx is the gradient
+ * of both x and res.  `x` of the backward is the saved `sum`. */
+int tf_add_layernorm_fwd(void* stream, int dtype, int param_dtype, int64_t rows, int64_t d,
+                         const void* x, int64_t ldx, const void* res, int64_t ldres,
+                         void* sum, int64_t ldsum, const void* gamma, const void* beta,
+                         float eps, void* y, int64_t ldy, float* mean, float* rstd);
+int tf_add_layernorm_bwd(void* stream, int dtype, int param_dtype, int64_t rows, int64_t d,
+                         const void* dy, int64_t lddy, const void* dsum, int64_t lddsum,
+                         const void* x, int64_t ldx, const void* gamma,
+                         const float* mean, const float* rstd,
+                         void* dx, int64_t lddx, void* dgamma, void* dbeta,
+                         float* partial, int64_t partial_bytes);
+
 /* Row softmax / its backward dx = y * (dy - sum(y*dy)); dtype f16/bf16/f32.
  * Replaces softmax_fwd / softmax_bwd (kernels/softmax.py:37-54, 95-111); the
  * backward writes a new buffer instead of overwriting grad_out. */

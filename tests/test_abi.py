@@ -23,7 +23,8 @@ def declared_functions():
 
 def test_header_declares_the_expected_surface():
     names = declared_functions()
-    for must in ["tf_gemm", "tf_attn_fwd", "tf_attn_bwd", "tf_layernorm_fwd", "tf_layernorm_bwd", "tf_softmax_fwd",
+    for must in ["tf_gemm", "tf_attn_fwd", "tf_attn_bwd", "tf_layernorm_fwd", "tf_layernorm_bwd", "tf_add_layernorm_fwd",
+                 "tf_add_layernorm_bwd", "tf_softmax_fwd",
                  "tf_softmax_bwd", "tf_cross_entropy_fwd", "tf_cross_entropy_bwd", "tf_colsum", "tf_relu_mask",
                  "tf_status_string", "tf_version"]:
         assert must in names
@@ -97,6 +98,17 @@ def test_row_kernels_reject_bad_arguments():
     assert lib.tf_layernorm_bwd(None, 0, 0, 4, 64, FAKE, 64, FAKE, 64, FAKE, FAKE, FAKE, FAKE, 64, FAKE, FAKE,
                                 None, 0) == -5
     assert lib.tf_layernorm_bwd_partial_bytes(8192, 1024) == 512 * 2 * 1024 * 4
+    # fused residual add: missing summand / sum buffer, short leading dimension, missing workspace
+    assert lib.tf_add_layernorm_fwd(None, 0, 0, 4, 64, FAKE, 64, None, 64, FAKE, 64, FAKE, FAKE, 1e-5, FAKE, 64, FAKE,
+                                    FAKE) == -1
+    assert lib.tf_add_layernorm_fwd(None, 0, 0, 4, 64, FAKE, 64, FAKE, 32, FAKE, 64, FAKE, FAKE, 1e-5, FAKE, 64, FAKE,
+                                    FAKE) == -1
+    assert lib.tf_add_layernorm_fwd(None, 2, 2, 4, 64, FAKE, 64, FAKE, 64, FAKE, 64, FAKE, FAKE, 1e-5, FAKE, 64, FAKE,
+                                    FAKE) == -2
+    assert lib.tf_add_layernorm_bwd(None, 0, 0, 4, 64, FAKE, 64, None, 64, FAKE, 64, FAKE, FAKE, FAKE, FAKE, 64, FAKE,
+                                    FAKE, FAKE, 1 << 20) == -1
+    assert lib.tf_add_layernorm_bwd(None, 0, 0, 4, 64, FAKE, 64, FAKE, 64, FAKE, 64, FAKE, FAKE, FAKE, FAKE, 64, FAKE,
+                                    FAKE, None, 0) == -5
     assert lib.tf_softmax_fwd(None, 0, 4, 0, FAKE, 64, FAKE, 64) == -1
     assert lib.tf_cross_entropy_fwd(None, 2, 4, 64, FAKE, 64, 0, 0, FAKE, FAKE, FAKE) == -2
     assert lib.tf_cross_entropy_bwd(None, 0, 4, 64, FAKE, 32, 0, 0, FAKE, FAKE, FAKE, 1, FAKE, 64, 0) == -1

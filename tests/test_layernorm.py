@@ -100,3 +100,64 @@ def test_layernorm_rejects_fp32_and_2d(dev):
     with pytest.raises(ValueError):
         T.layer_norm.apply(torch.zeros(4, 8, device=dev, dtype=h), torch.ones(8, device=dev, dtype=h),
                            torch.zeros(8, device=dev, dtype=h), 1e-5)
+
+
+@pytest.mark.parametrize("dims", [(2, 64, 768), (3, 77, 333), (1, 9, 5000), (4, 2048, 1024), (1, 3, 7)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_add_layernorm_equals_add_then_layernorm(dims, dtype, dev):
+    """The fused residual-add + LayerNorm node: forward results are bit-identical to an
+    elementwise addition followed by layer_norm (the sum is rounded to the 16-bit type
+    before the statistics); the backward adds the residual-stream gradient in fp32
+    before one rounding, so dx is compared with the fp32 oracle (atol 2e-2 fp16) and
+    with the two-node path."""
+    b, s, d = dims
+    g = torch.Generator().manual_seed(d)
+    x = torch.randn(b, s, d, generator=g).to(dtype)
+    br = (0.5 * torch.randn(b, s, d, generator=g)).to(dtype)
+    gamma, beta = torch.randn(d, generator=g), torch.randn(d, generator=g)   # fp32 master parameters
+    d_total = (0.5 * torch.randn(b, s, d, generator=g)).to(dtype)
+    d_y = torch.randn(b, s, d, generator=g).to(dtype)
+
+    def leaves():
+        return [t.to(dev).requires_grad_(True) for t in (x, br, gamma, beta)]
+
+    xd, bd, gd, btd = leaves()
+    total, y = T.add_layer_norm.apply(xd, bd, gd, btd, 1e-5)
+    torch.autograd.backward([total, y], [d_total.to(dev), d_y.to(dev)])
+    x2, b2, g2, bt2 = leaves()
+    total2 = x2 + b2
+    y2 = T.layer_norm.apply(total2, g2, bt2, 1e-5)
+    torch.autograd.backward([total2, y2], [d_total.to(dev), d_y.to(dev)])
+    assert torch.equal(total, total2) and torch.equal(y, y2)
+    assert xd.grad is not None and torch.equal(xd.grad, bd.grad)
+    # oracle: d(sum) = layernorm backward at the rounded sum + upstream gradient of the sum
+    dx, dg, db = R.layer_norm_bwd(total2.detach().cpu(), gamma, d_y, 1e-5)
+    want = dx.float() + d_total.float()
+    atol = 2e-2 if dtype == torch.float16 else 1.5e-1
+    assert_close(xd.grad, want, dtype, f"dx {dims}", atol=atol)
+    assert_close(xd.grad, x2.grad, dtype, f"dx vs two nodes {dims}", atol=atol)
+    lim = 1e-3 if dtype == torch.float16 else 8e-3
+    assert rel_l2(gd.grad, dg) < lim and rel_l2(btd.grad, db) < lim
+    assert torch.equal(gd.grad, g2.grad) and torch.equal(btd.grad, bt2.grad)
+
+
+def test_add_layernorm_unused_outputs(dev):
+    """Only one of the two outputs used downstream: the other's gradient arrives as None."""
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(2, 10, 256, generator=g).half().to(dev).requires_grad_(True)
+    br = torch.randn(2, 10, 256, generator=g).half().to(dev).requires_grad_(True)
+    gamma = torch.randn(256, generator=g).half().to(dev).requires_grad_(True)
+    beta = torch.randn(256, generator=g).half().to(dev).requires_grad_(True)
+    dy = torch.randn(2, 10, 256, generator=g).half().to(dev)
+    _, y = T.add_layer_norm.apply(x, br, gamma, beta, 1e-5)
+    y.backward(dy)
+    x2 = (x.detach() + br.detach()).requires_grad_(True)
+    g2, b2 = gamma.detach().clone().requires_grad_(True), beta.detach().clone().requires_grad_(True)
+    T.layer_norm.apply(x2, g2, b2, 1e-5).backward(dy)
+    assert torch.equal(x.grad, x2.grad) and torch.equal(br.grad, x2.grad) and torch.equal(gamma.grad, g2.grad)
+    x.grad = br.grad = gamma.grad = beta.grad = None
+    total, _ = T.add_layer_norm.apply(x, br, gamma, beta, 1e-5)
+    total.backward(dy)
+    assert torch.equal(x.grad, dy) and torch.equal(br.grad, dy) and gamma.grad is None
+    with pytest.raises(ValueError):
+        T.add_layer_norm.apply(x, br[:, :5], gamma, beta, 1e-5)

@@ -35,6 +35,10 @@ SIGNATURES = {
     "tf_layernorm_bwd": (_i, [_vp, _i, _i, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp,
                               _i64]),
     "tf_layernorm_bwd_partial_bytes": (_i64, [_i64, _i64]),
+    "tf_add_layernorm_fwd": (_i, [_vp, _i, _i, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _f, _vp, _i64,
+                                  _vp, _vp]),
+    "tf_add_layernorm_bwd": (_i, [_vp, _i, _i, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64,
+                                  _vp, _vp, _vp, _i64]),
     "tf_softmax_fwd": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _vp, _i64]),
     "tf_softmax_bwd": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64]),
     "tf_cross_entropy_fwd": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _i64, _i64, _vp, _vp, _vp]),

@@ -22,8 +22,13 @@ template <> __device__ __forceinline__ void load8<float>(const float* p, float (
 // ---------------------------------------------------------------------------
 // LayerNorm forward.  NV = 16-byte chunks per lane (row length <= NV*64*8).
 // ---------------------------------------------------------------------------
-template <typename T, typename TP, int NV>
+// With ADD the normalised row is s = x + res, rounded to T and also written to `sum`
+// (the residual stream after the addition); the statistics are those of the rounded s,
+// so the result equals an addition kernel followed by the plain forward.
+template <typename T, typename TP, int NV, bool ADD>
 __global__ __launch_bounds__(256) void ln_fwd_vec(int64_t rows, int d, const T* __restrict__ x, int64_t ldx,
+                                                   const T* __restrict__ res, int64_t ldres,
+                                                   T* __restrict__ sum, int64_t ldsum,
                                                    const TP* __restrict__ gamma, const TP* __restrict__ beta,
                                                    float eps, T* __restrict__ y, int64_t ldy,
                                                    float* __restrict__ mean_out, float* __restrict__ rstd_out) {
@@ -39,6 +44,15 @@ __global__ __launch_bounds__(256) void ln_fwd_vec(int64_t rows, int d, const T* 
     const int c = lane + i * 64;
     if (c < nchunk) {
       Chunk<T>::load(xr + c * 8, v[i]);
+      if (ADD) {
+        float r[8];
+        Chunk<T>::load(res + row * ldres + c * 8, r);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[i][e] += r[e];
+        const u32x4 packed = pack8<T>(v[i]);
+        st16(sum + row * ldsum + c * 8, packed);
+        unpack8<T>(packed, v[i]);
+      }
 #pragma unroll
       for (int e = 0; e < 8; ++e) s += v[i][e];
     } else {
@@ -75,8 +89,10 @@ __global__ __launch_bounds__(256) void ln_fwd_vec(int64_t rows, int d, const T* 
 
 // Any row length / alignment: scalar loads, three passes over the row (the
 // second and third come from cache).
-template <typename T, typename TP>
+template <typename T, typename TP, bool ADD>
 __global__ __launch_bounds__(256) void ln_fwd_any(int64_t rows, int d, const T* __restrict__ x, int64_t ldx,
+                                                   const T* __restrict__ res, int64_t ldres,
+                                                   T* __restrict__ sum, int64_t ldsum,
                                                    const TP* __restrict__ gamma, const TP* __restrict__ beta,
                                                    float eps, T* __restrict__ y, int64_t ldy,
                                                    float* __restrict__ mean_out, float* __restrict__ rstd_out) {
@@ -84,6 +100,12 @@ __global__ __launch_bounds__(256) void ln_fwd_any(int64_t rows, int d, const T* 
   const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
   if (row >= rows) return;
   const T* xr = x + row * ldx;
+  if (ADD) {
+    // every lane re-reads only the columns it wrote itself
+    T* sr = sum + row * ldsum;
+    for (int c = lane; c < d; c += 64) sr[c] = (T)((float)xr[c] + (float)res[row * ldres + c]);
+    xr = sr;
+  }
   float s = 0.f;
   for (int c = lane; c < d; c += 64) s += (float)xr[c];
   const float mean = wave_sum(s) / (float)d;
@@ -100,9 +122,14 @@ __global__ __launch_bounds__(256) void ln_fwd_any(int64_t rows, int d, const T* 
 // LayerNorm backward.  Wave w of workgroup b walks rows (b*4 + w) + k*4*grid.
 // dx is written per row; dgamma/dbeta partial sums stay in registers, are
 // summed over the 4 waves through LDS and land in partial[b][0|1][d].
+// The raw 16-byte chunks of the wave's next row are requested before the
+// cross-lane sums of the current row, so a wave always has loads in flight.
+// With ADD, dsum (the gradient that reaches the normalised tensor by another
+// path, e.g. along a residual stream) is added to dx before the rounding.
 // ---------------------------------------------------------------------------
-template <typename T, typename TP, int NV>
+template <typename T, typename TP, int NV, bool ADD>
 __global__ __launch_bounds__(256) void ln_bwd_vec(int64_t rows, int d, const T* __restrict__ dy, int64_t lddy,
+                                                   const T* __restrict__ dsum, int64_t lddsum,
                                                    const T* __restrict__ x, int64_t ldx,
                                                    const TP* __restrict__ gamma, const float* __restrict__ mean,
                                                    const float* __restrict__ rstd, T* __restrict__ dx,
@@ -120,20 +147,36 @@ __global__ __launch_bounds__(256) void ln_bwd_vec(int64_t rows, int d, const T* 
     if (c < nchunk) load8<TP>(gamma + c * 8, g[i]);
   }
   const float inv_d = 1.0f / (float)d;
-  for (int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + wave; row < rows;
-       row += (int64_t)gridDim.x * kRowsPerBlock) {
-    const float mu = mean[row], rs = rstd[row];
-    const T* xr = x + row * ldx;
-    const T* dyr = dy + row * lddy;
-    float xh[NV][8], gd[NV][8];
+  const int64_t stride = (int64_t)gridDim.x * kRowsPerBlock;
+  u32x4 raw_x[NV], raw_dy[NV], raw_ds[ADD ? NV : 1];
+  float mu_next = 0.f, rs_next = 0.f;
+  auto fetch = [&](int64_t row) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int c = lane + i * 64;
+      if (c < nchunk) {
+        raw_x[i] = ld16(x + row * ldx + c * 8);
+        raw_dy[i] = ld16(dy + row * lddy + c * 8);
+        if (ADD) raw_ds[i] = ld16(dsum + row * lddsum + c * 8);
+      }
+    }
+    mu_next = mean[row];
+    rs_next = rstd[row];
+  };
+  int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + wave;
+  if (row < rows) fetch(row);
+  for (; row < rows; row += stride) {
+    const float mu = mu_next, rs = rs_next;
+    float xh[NV][8], gd[NV][8], ds[ADD ? NV : 1][8];
     float s1 = 0.f, s2 = 0.f;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int c = lane + i * 64;
       if (c < nchunk) {
         float xv[8], dv[8];
-        Chunk<T>::load(xr + c * 8, xv);
-        Chunk<T>::load(dyr + c * 8, dv);
+        unpack8<T>(raw_x[i], xv);
+        unpack8<T>(raw_dy[i], dv);
+        if (ADD) unpack8<T>(raw_ds[i], ds[i]);
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           xh[i][e] = (xv[e] - mu) * rs;
@@ -148,6 +191,7 @@ __global__ __launch_bounds__(256) void ln_bwd_vec(int64_t rows, int d, const T* 
         for (int e = 0; e < 8; ++e) { xh[i][e] = 0.f; gd[i][e] = 0.f; }
       }
     }
+    if (row + stride < rows) fetch(row + stride);
     const float c1 = wave_sum(s1) * inv_d;
     const float c2 = wave_sum(s2) * inv_d;
     T* dxr = dx + row * lddx;
@@ -157,7 +201,10 @@ __global__ __launch_bounds__(256) void ln_bwd_vec(int64_t rows, int d, const T* 
       if (c < nchunk) {
         float o[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) o[e] = (gd[i][e] - xh[i][e] * c1 - c2) * rs;
+        for (int e = 0; e < 8; ++e) {
+          o[e] = (gd[i][e] - xh[i][e] * c1 - c2) * rs;
+          if (ADD) o[e] += ds[i][e];
+        }
         Chunk<T>::store(dxr + c * 8, o);
       }
     }
@@ -181,8 +228,9 @@ __global__ __launch_bounds__(256) void ln_bwd_vec(int64_t rows, int d, const T* 
   }
 }
 
-template <typename T, typename TP>
+template <typename T, typename TP, bool ADD>
 __global__ __launch_bounds__(256) void ln_bwd_any(int64_t rows, int d, const T* __restrict__ dy, int64_t lddy,
+                                                   const T* __restrict__ dsum, int64_t lddsum,
                                                    const T* __restrict__ x, int64_t ldx,
                                                    const TP* __restrict__ gamma, const float* __restrict__ mean,
                                                    const float* __restrict__ rstd, T* __restrict__ dx,
@@ -217,24 +265,37 @@ __global__ __launch_bounds__(256) void ln_bwd_any(int64_t rows, int d, const T* 
     T* dxr = dx + row * lddx;
     for (int c = threadIdx.x; c < d; c += 256) {
       const float xh = ((float)xr[c] - mu) * rs, gd = (float)dyr[c] * (float)gamma[c];
-      dxr[c] = (T)((gd - xh * c1 - c2) * rs);
+      float o = (gd - xh * c1 - c2) * rs;
+      if (ADD) o += (float)dsum[row * lddsum + c];
+      dxr[c] = (T)o;
     }
   }
 }
 
 // Second stage over partial viewed as a [nparts][2d] matrix (dgamma columns then
 // dbeta columns): workgroup = 16 columns x 16 row slices, slices summed in a
-// fixed order through LDS.
+// fixed order through LDS.  Four independent running sums per thread keep
+// several loads in flight.
 template <typename T>
 __global__ __launch_bounds__(256) void ln_bwd_reduce(int nparts, int d, const float* __restrict__ partial,
                                                       T* __restrict__ dgamma, T* __restrict__ dbeta) {
   __shared__ float red[16][17];
   const int cl = threadIdx.x & 15, slice = threadIdx.x >> 4;
   const int col = blockIdx.x * 16 + cl;  // 0 .. 2d-1
-  float a = 0.f;
-  if (col < 2 * d)
-    for (int p = slice; p < nparts; p += 16) a += partial[(int64_t)p * 2 * d + col];
-  red[slice][cl] = a;
+  float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+  if (col < 2 * d) {
+    const float* src = partial + col;
+    const int64_t ld = 2 * (int64_t)d;
+    int p = slice;
+    for (; p + 48 < nparts; p += 64) {
+      a0 += src[(int64_t)p * ld];
+      a1 += src[(int64_t)(p + 16) * ld];
+      a2 += src[(int64_t)(p + 32) * ld];
+      a3 += src[(int64_t)(p + 48) * ld];
+    }
+    for (; p < nparts; p += 16) a0 += src[(int64_t)p * ld];
+  }
+  red[slice][cl] = (a0 + a1) + (a2 + a3);
   __syncthreads();
   if (slice == 0 && col < 2 * d) {
     float s = 0.f;
@@ -366,24 +427,27 @@ static int pick_nv(int64_t nchunk) {
   return 0;
 }
 
-template <typename T, typename TP>
-static int ln_fwd_launch(hipStream_t st, int64_t rows, int64_t d, const void* x, int64_t ldx, const void* gamma,
-                         const void* beta, float eps, void* y, int64_t ldy, float* mean, float* rstd) {
+template <typename T, typename TP, bool ADD>
+static int ln_fwd_launch(hipStream_t st, int64_t rows, int64_t d, const void* x, int64_t ldx, const void* res,
+                         int64_t ldres, void* sum, int64_t ldsum, const void* gamma, const void* beta, float eps,
+                         void* y, int64_t ldy, float* mean, float* rstd) {
   const dim3 grid((unsigned)ceil_div(rows, kRowsPerBlock)), block(256);
-  const bool vec = row_vectorizable<T>(x, d, ldx) && row_vectorizable<T>(y, d, ldy) && aligned16(gamma) &&
-                   aligned16(beta);
+  bool vec = row_vectorizable<T>(x, d, ldx) && row_vectorizable<T>(y, d, ldy) && aligned16(gamma) && aligned16(beta);
+  if (ADD) vec = vec && row_vectorizable<T>(res, d, ldres) && row_vectorizable<T>(sum, d, ldsum);
   const int nv = vec ? pick_nv(d / 8) : 0;
-#define LN_FWD(NV)                                                                                           \
-  ln_fwd_vec<T, TP, NV><<<grid, block, 0, st>>>(rows, (int)d, (const T*)x, ldx, (const TP*)gamma, (const TP*)beta, \
-                                            eps, (T*)y, ldy, mean, rstd)
+#define LN_FWD(NV)                                                                                             \
+  ln_fwd_vec<T, TP, NV, ADD><<<grid, block, 0, st>>>(rows, (int)d, (const T*)x, ldx, (const T*)res, ldres, (T*)sum, \
+                                                     ldsum, (const TP*)gamma, (const TP*)beta, eps, (T*)y, ldy, mean, \
+                                                     rstd)
   switch (nv) {
     case 1: LN_FWD(1); break;
     case 2: LN_FWD(2); break;
     case 4: LN_FWD(4); break;
     case 8: LN_FWD(8); break;
     default:
-      ln_fwd_any<T, TP><<<grid, block, 0, st>>>(rows, (int)d, (const T*)x, ldx, (const TP*)gamma, (const TP*)beta, eps,
-                                            (T*)y, ldy, mean, rstd);
+      ln_fwd_any<T, TP, ADD><<<grid, block, 0, st>>>(rows, (int)d, (const T*)x, ldx, (const T*)res, ldres, (T*)sum,
+                                                     ldsum, (const TP*)gamma, (const TP*)beta, eps, (T*)y, ldy, mean,
+                                                     rstd);
   }
 #undef LN_FWD
   TF_CHECK_LAUNCH();
@@ -395,26 +459,29 @@ static int ln_bwd_parts(int64_t rows) {
   return (int)(g < 512 ? g : 512);
 }
 
-template <typename T, typename TP>
-static int ln_bwd_launch(hipStream_t st, int64_t rows, int64_t d, const void* dy, int64_t lddy, const void* x,
-                         int64_t ldx, const void* gamma, const float* mean, const float* rstd, void* dx,
-                         int64_t lddx, void* dgamma, void* dbeta, float* partial) {
+template <typename T, typename TP, bool ADD>
+static int ln_bwd_launch(hipStream_t st, int64_t rows, int64_t d, const void* dy, int64_t lddy, const void* dsum,
+                         int64_t lddsum, const void* x, int64_t ldx, const void* gamma, const float* mean,
+                         const float* rstd, void* dx, int64_t lddx, void* dgamma, void* dbeta, float* partial) {
   const int parts = ln_bwd_parts(rows);
-  const bool vec = row_vectorizable<T>(x, d, ldx) && row_vectorizable<T>(dy, d, lddy) &&
-                   row_vectorizable<T>(dx, d, lddx) && aligned16(gamma);
+  bool vec = row_vectorizable<T>(x, d, ldx) && row_vectorizable<T>(dy, d, lddy) && row_vectorizable<T>(dx, d, lddx) &&
+             aligned16(gamma);
+  if (ADD) vec = vec && row_vectorizable<T>(dsum, d, lddsum);
   const int nv = vec ? pick_nv(d / 8) : 0;
   const size_t lds = (size_t)4 * d * sizeof(float);
-#define LN_BWD(NV)                                                                                          \
-  ln_bwd_vec<T, TP, NV><<<dim3(parts), dim3(256), lds, st>>>(rows, (int)d, (const T*)dy, lddy, (const T*)x, ldx, \
-                                                             (const TP*)gamma, mean, rstd, (T*)dx, lddx, partial)
+#define LN_BWD(NV)                                                                                                \
+  ln_bwd_vec<T, TP, NV, ADD><<<dim3(parts), dim3(256), lds, st>>>(rows, (int)d, (const T*)dy, lddy, (const T*)dsum,   \
+                                                                  lddsum, (const T*)x, ldx, (const TP*)gamma, mean, \
+                                                                  rstd, (T*)dx, lddx, partial)
   switch (nv) {
     case 1: LN_BWD(1); break;
     case 2: LN_BWD(2); break;
     case 4: LN_BWD(4); break;
     case 8: LN_BWD(8); break;
     default:
-      ln_bwd_any<T, TP><<<dim3(parts), dim3(256), 0, st>>>(rows, (int)d, (const T*)dy, lddy, (const T*)x, ldx,
-                                                           (const TP*)gamma, mean, rstd, (T*)dx, lddx, partial);
+      ln_bwd_any<T, TP, ADD><<<dim3(parts), dim3(256), 0, st>>>(rows, (int)d, (const T*)dy, lddy, (const T*)dsum,
+                                                                lddsum, (const T*)x, ldx, (const TP*)gamma, mean,
+                                                                rstd, (T*)dx, lddx, partial);
   }
 #undef LN_BWD
   TF_CHECK_LAUNCH();
@@ -472,22 +539,37 @@ static bool bad_rows(int64_t rows, int64_t n, int64_t ld) {
 
 using namespace tfa;
 
-extern "C" int tf_layernorm_fwd(void* stream, int dtype, int param_dtype, int64_t rows, int64_t d, const void* x,
-                                int64_t ldx, const void* gamma, const void* beta, float eps, void* y, int64_t ldy,
-                                float* mean, float* rstd) {
+template <bool ADD>
+static int ln_fwd_entry(void* stream, int dtype, int param_dtype, int64_t rows, int64_t d, const void* x, int64_t ldx,
+                        const void* res, int64_t ldres, void* sum, int64_t ldsum, const void* gamma,
+                        const void* beta, float eps, void* y, int64_t ldy, float* mean, float* rstd) {
   if (!x || !gamma || !beta || !y || !mean || !rstd) return TF_EINVAL;
+  if (ADD && (!res || !sum || ldres < d || ldsum < d)) return TF_EINVAL;
   if (bad_rows(rows, d, ldx) || ldy < d) return TF_EINVAL;
   if (rows == 0) return TF_OK;
   hipStream_t st = (hipStream_t)stream;
   if (param_dtype != dtype && param_dtype != TF_F32) return TF_EDTYPE;
-  const bool pf = param_dtype == TF_F32;
-  if (dtype == TF_F16)
-    return pf ? ln_fwd_launch<f16, float>(st, rows, d, x, ldx, gamma, beta, eps, y, ldy, mean, rstd)
-              : ln_fwd_launch<f16, f16>(st, rows, d, x, ldx, gamma, beta, eps, y, ldy, mean, rstd);
-  if (dtype == TF_BF16)
-    return pf ? ln_fwd_launch<bf16, float>(st, rows, d, x, ldx, gamma, beta, eps, y, ldy, mean, rstd)
-              : ln_fwd_launch<bf16, bf16>(st, rows, d, x, ldx, gamma, beta, eps, y, ldy, mean, rstd);
+#define LN_FWD_GO(T, TP) \
+  return ln_fwd_launch<T, TP, ADD>(st, rows, d, x, ldx, res, ldres, sum, ldsum, gamma, beta, eps, y, ldy, mean, rstd)
+  if (dtype == TF_F16) { if (param_dtype == TF_F32) LN_FWD_GO(f16, float); else LN_FWD_GO(f16, f16); }
+  if (dtype == TF_BF16) { if (param_dtype == TF_F32) LN_FWD_GO(bf16, float); else LN_FWD_GO(bf16, bf16); }
+#undef LN_FWD_GO
   return TF_EDTYPE;
+}
+
+extern "C" int tf_layernorm_fwd(void* stream, int dtype, int param_dtype, int64_t rows, int64_t d, const void* x,
+                                int64_t ldx, const void* gamma, const void* beta, float eps, void* y, int64_t ldy,
+                                float* mean, float* rstd) {
+  return ln_fwd_entry<false>(stream, dtype, param_dtype, rows, d, x, ldx, nullptr, 0, nullptr, 0, gamma, beta, eps, y,
+                             ldy, mean, rstd);
+}
+
+extern "C" int tf_add_layernorm_fwd(void* stream, int dtype, int param_dtype, int64_t rows, int64_t d, const void* x,
+                                    int64_t ldx, const void* res, int64_t ldres, void* sum, int64_t ldsum,
+                                    const void* gamma, const void* beta, float eps, void* y, int64_t ldy, float* mean,
+                                    float* rstd) {
+  return ln_fwd_entry<true>(stream, dtype, param_dtype, rows, d, x, ldx, res, ldres, sum, ldsum, gamma, beta, eps, y,
+                            ldy, mean, rstd);
 }
 
 extern "C" int64_t tf_layernorm_bwd_partial_bytes(int64_t rows, int64_t d) {
@@ -495,22 +577,40 @@ extern "C" int64_t tf_layernorm_bwd_partial_bytes(int64_t rows, int64_t d) {
   return (int64_t)ln_bwd_parts(rows) * 2 * d * (int64_t)sizeof(float);
 }
 
-extern "C" int tf_layernorm_bwd(void* stream, int dtype, int param_dtype, int64_t rows, int64_t d, const void* dy,
-                                int64_t lddy,
-                                const void* x, int64_t ldx, const void* gamma, const float* mean,
-                                const float* rstd, void* dx, int64_t lddx, void* dgamma, void* dbeta,
-                                float* partial, int64_t partial_bytes) {
+template <bool ADD>
+static int ln_bwd_entry(void* stream, int dtype, int param_dtype, int64_t rows, int64_t d, const void* dy,
+                        int64_t lddy, const void* dsum, int64_t lddsum, const void* x, int64_t ldx,
+                        const void* gamma, const float* mean, const float* rstd, void* dx, int64_t lddx,
+                        void* dgamma, void* dbeta, float* partial, int64_t partial_bytes) {
   if (!dy || !x || !gamma || !mean || !rstd || !dx || !dgamma || !dbeta) return TF_EINVAL;
+  if (ADD && (!dsum || lddsum < d)) return TF_EINVAL;
   if (bad_rows(rows, d, ldx) || lddy < d || lddx < d || rows == 0) return TF_EINVAL;
   if (!partial || partial_bytes < tf_layernorm_bwd_partial_bytes(rows, d)) return TF_EWORKSPACE;
   hipStream_t st = (hipStream_t)stream;
   if (param_dtype != dtype && param_dtype != TF_F32) return TF_EDTYPE;
-#define LN_BWD_GO(T, TP) \
-  return ln_bwd_launch<T, TP>(st, rows, d, dy, lddy, x, ldx, gamma, mean, rstd, dx, lddx, dgamma, dbeta, partial)
+#define LN_BWD_GO(T, TP)                                                                                          \
+  return ln_bwd_launch<T, TP, ADD>(st, rows, d, dy, lddy, dsum, lddsum, x, ldx, gamma, mean, rstd, dx, lddx, dgamma, \
+                                   dbeta, partial)
   if (dtype == TF_F16) { if (param_dtype == TF_F32) LN_BWD_GO(f16, float); else LN_BWD_GO(f16, f16); }
   if (dtype == TF_BF16) { if (param_dtype == TF_F32) LN_BWD_GO(bf16, float); else LN_BWD_GO(bf16, bf16); }
 #undef LN_BWD_GO
   return TF_EDTYPE;
+}
+
+extern "C" int tf_layernorm_bwd(void* stream, int dtype, int param_dtype, int64_t rows, int64_t d, const void* dy,
+                                int64_t lddy, const void* x, int64_t ldx, const void* gamma, const float* mean,
+                                const float* rstd, void* dx, int64_t lddx, void* dgamma, void* dbeta,
+                                float* partial, int64_t partial_bytes) {
+  return ln_bwd_entry<false>(stream, dtype, param_dtype, rows, d, dy, lddy, nullptr, 0, x, ldx, gamma, mean, rstd, dx,
+                             lddx, dgamma, dbeta, partial, partial_bytes);
+}
+
+extern "C" int tf_add_layernorm_bwd(void* stream, int dtype, int param_dtype, int64_t rows, int64_t d, const void* dy,
+                                    int64_t lddy, const void* dsum, int64_t lddsum, const void* x, int64_t ldx,
+                                    const void* gamma, const float* mean, const float* rstd, void* dx, int64_t lddx,
+                                    void* dgamma, void* dbeta, float* partial, int64_t partial_bytes) {
+  return ln_bwd_entry<true>(stream, dtype, param_dtype, rows, d, dy, lddy, dsum, lddsum, x, ldx, gamma, mean, rstd, dx,
+                            lddx, dgamma, dbeta, partial, partial_bytes);
 }
 
 extern "C" int tf_softmax_fwd(void* stream, int dtype, int64_t rows, int64_t cols, const void* x, int64_t ldx,

@@ -279,6 +279,47 @@ def layernorm_bwd(grad_out, x, alpha, mean, rstd):
     return dx, da, db
 
 
+def add_layernorm_fwd(x, res, alpha, beta, eps):
+    """-> (sum, y, mean, rstd) with sum = x + res and y = layernorm(sum), one kernel for the
+    residual addition (reference transformer.py:245-246, :250) and the LayerNorm after it."""
+    _check_ln(x, alpha.shape[0])
+    if res.shape != x.shape or res.dtype != x.dtype:
+        raise ValueError("the two summands must have the same shape and dtype")
+    if alpha.dtype != beta.dtype or alpha.dtype not in (x.dtype, torch.float32):
+        raise TypeError("LayerNorm parameters must have the input's dtype or be float32")
+    require_cuda(res, alpha, beta)
+    x2, rows, d = _rows2d(x)
+    r2, _, _ = _rows2d(res)
+    total = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    y = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    mean = torch.empty((rows,), dtype=torch.float32, device=x.device)
+    rstd = torch.empty((rows,), dtype=torch.float32, device=x.device)
+    check(load().tf_add_layernorm_fwd(stream_ptr(), dtype_code(x.dtype), dtype_code(alpha.dtype), rows, d,
+                                      x2.data_ptr(), d, r2.data_ptr(), d, total.data_ptr(), d,
+                                      alpha.contiguous().data_ptr(), beta.contiguous().data_ptr(), float(eps),
+                                      y.data_ptr(), d, mean.data_ptr(), rstd.data_ptr()))
+    return total, y, mean, rstd
+
+
+def add_layernorm_bwd(grad_out, grad_sum, total, alpha, mean, rstd):
+    """-> (dx, dalpha, dbeta): dx = layernorm backward of grad_out at the saved sum, plus
+    grad_sum (the gradient of the sum arriving along the residual stream)."""
+    lib = load()
+    x2, rows, d = _rows2d(total)
+    g2, _, _ = _rows2d(grad_out)
+    s2, _, _ = _rows2d(grad_sum)
+    dx = torch.empty(total.shape, dtype=total.dtype, device=total.device)
+    da = torch.empty((d,), dtype=alpha.dtype, device=total.device)
+    db = torch.empty((d,), dtype=alpha.dtype, device=total.device)
+    pb = lib.tf_layernorm_bwd_partial_bytes(rows, d)
+    part = torch.empty(pb, dtype=torch.uint8, device=total.device)
+    check(lib.tf_add_layernorm_bwd(stream_ptr(), dtype_code(total.dtype), dtype_code(alpha.dtype), rows, d,
+                                   g2.data_ptr(), d, s2.data_ptr(), d, x2.data_ptr(), d,
+                                   alpha.contiguous().data_ptr(), mean.data_ptr(), rstd.data_ptr(), dx.data_ptr(), d,
+                                   da.data_ptr(), db.data_ptr(), part.data_ptr(), pb))
+    return dx, da, db
+
+
 # --------------------------------------------------------------------------- softmax
 def softmax_fwd(x):
     """Row softmax over the last dim (reference kernels/softmax.py:37-54)."""

@@ -3,7 +3,7 @@ reference's tritonformer/layernorm.py."""
 from torch.autograd import Function
 
 from ._amp import amp_bwd, amp_fwd
-from .kernels import layernorm_bwd, layernorm_fwd
+from .kernels import add_layernorm_bwd, add_layernorm_fwd, layernorm_bwd, layernorm_fwd
 
 
 class LayerNorm(Function):
@@ -21,3 +21,31 @@ class LayerNorm(Function):
         input, alpha, mean, rstd = ctx.saved_tensors
         grad_input, grad_alpha, grad_beta = layernorm_bwd(grad_output, input, alpha, mean, rstd)
         return grad_input, grad_alpha, grad_beta, None
+
+
+class AddLayerNorm(Function):
+    """``apply(x, branch, alpha, beta, eps) -> (x + branch, layernorm(x + branch))``: the
+    residual addition of the reference's TransformerLayer (transformer.py:245-246, :250)
+    and the LayerNorm that follows it as one graph node with one kernel per direction.
+    Both outputs are differentiable; the backward returns one tensor as the gradient of
+    both summands."""
+
+    @staticmethod
+    @amp_fwd(keep=(2, 3))
+    def forward(ctx, x, branch, alpha, beta, eps):
+        total, x_ln, mean, rstd = add_layernorm_fwd(x, branch, alpha, beta, eps)
+        ctx.save_for_backward(total, alpha, mean, rstd)
+        ctx.set_materialize_grads(False)  # an unused output arrives as None, not as zeros
+        return total, x_ln
+
+    @staticmethod
+    @amp_bwd
+    def backward(ctx, grad_total, grad_ln):
+        total, alpha, mean, rstd = ctx.saved_tensors
+        if grad_ln is None:  # only the sum was used downstream
+            return grad_total, grad_total, None, None, None
+        if grad_total is None:
+            dx, da, db = layernorm_bwd(grad_ln, total, alpha, mean, rstd)
+        else:
+            dx, da, db = add_layernorm_bwd(grad_ln, grad_total, total, alpha, mean, rstd)
+        return dx, dx, da, db, None

@@ -19,6 +19,7 @@ import torch
 import torch.nn as nn
 
 from . import (
+    add_layer_norm,
     fast_causal_attention,
     fast_causal_attention_qkvpacked,
     fast_causal_attention_with_bias,
@@ -75,6 +76,11 @@ FUSE_QKV = True
 # True: the MLP block is one autograd node (ReLU gradient mask fused into a GEMM write-out);
 # False: two Linear modules as in the reference (transformer.py:214-217).
 FUSE_MLP = True
+# True: every residual addition runs inside the LayerNorm kernel that consumes its result
+# (forward), and the residual-stream gradient is added inside that LayerNorm's backward
+# kernel: no separate elementwise addition kernels.  False: `residual + hidden_states`
+# as the reference writes it (transformer.py:245-250).
+FUSE_ADD_LN = True
 
 
 def _weights_init(model: nn.Module, num_layers: int) -> None:
@@ -170,6 +176,20 @@ class TransformerLayer(nn.Module):
         hidden_states = hidden_states + self.attention(self.input_layernorm(hidden_states), attn_bias)
         return hidden_states + self.mlp(self.post_attention_layernorm(hidden_states))
 
+    def forward_deferred(self, hidden_states: torch.Tensor, pending: Optional[torch.Tensor],
+                         attn_bias: Optional[torch.Tensor] = None):
+        """Same block with the additions folded into the LayerNorms: takes the residual stream
+        and a branch output not yet added to it (None for the first block), returns the stream
+        after the attention residual and this block's MLP output, still to be added."""
+        ln1, ln2 = self.input_layernorm, self.post_attention_layernorm
+        if pending is None:
+            normed = ln1(hidden_states)
+        else:
+            hidden_states, normed = add_layer_norm.apply(hidden_states, pending, ln1.weight, ln1.bias, ln1.eps)
+        attn_out = self.attention(normed, attn_bias)
+        hidden_states, normed = add_layer_norm.apply(hidden_states, attn_out, ln2.weight, ln2.bias, ln2.eps)
+        return hidden_states, self.mlp(normed)
+
 
 class Transformer(nn.Module):
     """Decoder stack + LM head + shifted cross-entropy (reference transformer.py:254-346)."""
@@ -211,9 +231,16 @@ class Transformer(nn.Module):
             hidden_states = hidden_states.to(torch.get_autocast_dtype("cuda"))
             if attn_bias is not None:
                 attn_bias = attn_bias.to(torch.get_autocast_dtype("cuda"))
-        for layer in self.layer_list:
-            hidden_states = layer(hidden_states, attn_bias)
-        hidden_states = self.final_layernorm(hidden_states)
+        if FUSE_ADD_LN and len(self.layer_list) > 0:
+            pending = None
+            for layer in self.layer_list:
+                hidden_states, pending = layer.forward_deferred(hidden_states, pending, attn_bias)
+            ln = self.final_layernorm
+            _, hidden_states = add_layer_norm.apply(hidden_states, pending, ln.weight, ln.bias, ln.eps)
+        else:
+            for layer in self.layer_list:
+                hidden_states = layer(hidden_states, attn_bias)
+            hidden_states = self.final_layernorm(hidden_states)
         logits_lm = self.logits_out(hidden_states)
         if labels is None:
             return logits_lm
