@@ -86,6 +86,20 @@ int tf_gemm_out(void* stream, int dtype, int out_dtype, int layout_a, int layout
                 void* C, int64_t ldc, const void* bias, int relu,
                 const void* mask_act, int64_t ld_mask,
                 void* workspace, int64_t workspace_bytes);
+/* As tf_gemm_out, with C split into N / chunk_n column blocks that are separate
+ * (M, chunk_n) matrices of leading dimension ldc, `chunk_stride` elements apart:
+ * element (m, n) is stored at C[(n / chunk_n) * chunk_stride + m * ldc + n % chunk_n].
+ * Used for the weight gradient of the q, k and v projections computed as ONE
+ * product x^T . d(qkv) (the three dW products of tritonformer/linear.py:25 for
+ * transformer.py:158-160): every projection gets its own contiguous gradient.
+ * chunk_n = 0 means one matrix; otherwise chunk_n divides N and chunk_n,
+ * chunk_stride are multiples of 8. */
+int tf_gemm_out_chunked(void* stream, int dtype, int out_dtype, int layout_a, int layout_b,
+                        int64_t M, int64_t N, int64_t K,
+                        const void* A, int64_t lda, const void* B, int64_t ldb,
+                        void* C, int64_t ldc, int64_t chunk_n, int64_t chunk_stride,
+                        const void* bias, int relu, const void* mask_act, int64_t ld_mask,
+                        void* workspace, int64_t workspace_bytes);
 int64_t tf_gemm_workspace_bytes(int layout_a, int layout_b, int64_t M, int64_t N, int64_t K);
 /* Diagnostic, no counterpart in the reference (whose Triton autotuner picks
  * tiles per shape, kernels/gemm.py:15-79): force tile configuration `cfg`
@@ -169,6 +183,16 @@ int tf_add_layernorm_bwd(void* stream, int dtype, int param_dtype, int64_t rows,
                          const float* mean, const float* rstd,
                          void* dx, int64_t lddx, void* dgamma, void* dbeta,
                          float* partial, int64_t partial_bytes);
+
+/* dst[r, j*cols + c] = (dst_dtype) srcs[j][r*ld_src + c] for j < count (count <= 4):
+ * `count` (rows, cols) matrices of src_dtype (TF_F32, or dst_dtype) converted to
+ * 16 bits and laid side by side in one (rows, count*cols) matrix, one launch.
+ * Builds the 16-bit (d, 3d) operand of the packed q/k/v projection from the three
+ * master weights; stands for the three per-parameter casts torch.autocast makes
+ * for the reference's three projections (transformer.py:158-160).
+ * `srcs`: HOST array of `count` device pointers. */
+int tf_cast_pack(void* stream, int src_dtype, int dst_dtype, int count, int64_t rows, int64_t cols,
+                 const void* const* srcs, int64_t ld_src, void* dst, int64_t ld_dst);
 
 /* Row softmax / its backward dx = y * (dy - sum(y*dy)); dtype f16/bf16/f32.
  * Replaces softmax_fwd / softmax_bwd (kernels/softmax.py:37-54, 95-111); the

@@ -70,6 +70,19 @@ def test_gemm_rejects_bad_arguments():
     assert lib.tf_gemm_out(None, 0, 1, 0, 1, 64, 64, 64, *out_tail) == -2                       # bf16 out of fp16 in
     assert lib.tf_gemm_out(None, 0, 0, 0, 1, 64, 64, 64, FAKE, 64, FAKE, 64, FAKE, 64, None, 1, FAKE, 64,
                            None, 0) == -1                                                        # mask with ReLU
+    # column-block output: blocks must divide N, be multiples of 8 wide and not overlap
+    def chunked(chunk_n, chunk_stride, ldc=32):
+        return lib.tf_gemm_out_chunked(None, 0, 2, 1, 1, 64, 96, 64, FAKE, 64, FAKE, 96, FAKE, ldc, chunk_n,
+                                       chunk_stride, None, 0, None, 0, None, 0)
+    assert chunked(36, 64 * 32) == -4 and chunked(32, 63 * 32) == -4 and chunked(32, 64 * 32, ldc=24) == -4
+    assert chunked(-1, 0) == -1
+    import ctypes
+    ptrs = (ctypes.c_void_p * 3)(FAKE, FAKE, FAKE)
+    assert lib.tf_cast_pack(None, 2, 0, 5, 8, 8, ptrs, 8, FAKE, 40) == -1          # more than 4 sources
+    assert lib.tf_cast_pack(None, 2, 0, 3, 8, 8, ptrs, 8, FAKE, 16) == -1          # destination rows too short
+    assert lib.tf_cast_pack(None, 1, 0, 3, 8, 8, ptrs, 8, FAKE, 24) == -2          # bf16 -> fp16
+    assert lib.tf_cast_pack(None, 2, 2, 3, 8, 8, ptrs, 8, FAKE, 24) == -2          # fp32 destination
+    assert lib.tf_cast_pack(None, 2, 0, 3, 0, 8, ptrs, 8, FAKE, 24) == 0           # nothing to do
 
 
 def test_attention_rejects_bad_shapes():

@@ -212,3 +212,68 @@ def test_fused_mlp_equals_two_functions(dims, use_bias, dev):
     y_ref = R.linear(R.linear(x.cpu(), w1.cpu(), b1.cpu() if use_bias else None, True).half(), w2.cpu(),
                      b2.cpu() if use_bias else None)
     assert_close(ya, y_ref, name="mlp y", atol=2e-2)
+
+
+@pytest.mark.parametrize("dims", [(2, 77, 328, 136), (4, 2048, 1024, 1024), (1, 64, 64, 8)])
+@pytest.mark.parametrize("master", [False, True])
+def test_packed_projections_equal_separate_functions(dims, master, dev):
+    """linear_no_bias_packed(x, Wq, Wk, Wv) against three linear_no_bias calls: the
+    forward is the same arithmetic per element (bitwise equal), the weight gradients
+    are the same products summed in fp32 (equal up to summation order); dX sums one contraction of length 3*out instead of three rounded partial
+    results, so it is compared with the fp32 oracle at the linear tolerance.
+    `master`: fp32 weights under autocast (fp32 gradients straight from the accumulators)."""
+    b, m, n, k = dims
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(b, m, n, generator=g).half()
+    ws = [(torch.randn(n, k, generator=g) / n ** 0.5) for _ in range(3)]
+    if not master:
+        ws = [w.half() for w in ws]
+    dy = torch.randn(b, m, 3 * k, generator=g).half()
+
+    def run(packed):
+        xd = x.to(dev).requires_grad_(True)
+        wd = [w.to(dev).requires_grad_(True) for w in ws]
+        with torch.autocast("cuda", dtype=torch.float16, enabled=master):
+            if packed:
+                y = T.linear_no_bias_packed.apply(xd, *wd)
+            else:
+                y = torch.cat([T.linear_no_bias.apply(xd, w) for w in wd], dim=-1)
+        y.backward(dy.to(dev))
+        return y, xd.grad, [w.grad for w in wd]
+
+    y1, dx1, dw1 = run(True)
+    y0, dx0, dw0 = run(False)
+    assert torch.equal(y1, y0)
+    for a, c in zip(dw1, dw0):
+        assert a.is_contiguous() and a.dtype == (torch.float32 if master else torch.float16)
+        # same products; the contraction over B*S may be split differently for the (in, 3*out)
+        # problem than for (in, out), which changes the fp32 summation order only
+        assert rel_l2(a, c) < (1e-5 if master else 1e-3)
+    w16 = torch.cat([w.half() for w in ws], dim=1)
+    dx_ref, _, _ = R.linear_bwd(x, w16, dy, act=None, with_bias=False)
+    assert_close(dx1, dx_ref, torch.float16, f"packed dx {dims}", atol=2e-2)
+
+
+def test_cast_pack_and_chunked_weight_gradient(dev):
+    from tritonformer_amd import kernels as K
+
+    g = torch.Generator().manual_seed(2)
+    ws = [torch.randn(40, 24, generator=g).to(dev) for _ in range(3)]
+    for dt in (torch.float16, torch.bfloat16):
+        assert torch.equal(K.cast_pack(ws, dt), torch.cat([w.to(dt) for w in ws], dim=1))
+        assert torch.equal(K.cast_pack([w.to(dt) for w in ws[:2]], dt), torch.cat([w.to(dt) for w in ws[:2]], dim=1))
+    odd = [torch.randn(5, 7, generator=g).to(dev) for _ in range(4)]     # no 16-byte chunks: element path
+    assert torch.equal(K.cast_pack(odd, torch.float16), torch.cat([w.half() for w in odd], dim=1))
+    with pytest.raises(ValueError):
+        K.cast_pack(ws + ws, torch.float16)
+    with pytest.raises(TypeError):
+        K.cast_pack([w.half() for w in ws], torch.bfloat16)
+    x = torch.randn(2, 300, 72, generator=g).half().to(dev)
+    dy = torch.randn(2, 300, 96, generator=g).half().to(dev)
+    for od in (None, torch.float32):
+        whole = K.mm_dw(x, dy, out_dtype=od)
+        parts = K.mm_dw(x, dy, out_dtype=od, chunks=3)
+        assert parts.shape == (3, 72, 32)
+        assert torch.equal(torch.cat(list(parts), dim=1), whole)
+    with pytest.raises(ValueError):
+        K.mm_dw(x, dy, chunks=5)

@@ -15,4 +15,5 @@ from .linear import LinearBiasReLU as linear_fused_bias_relu
 from .linear import LinearNoBias as linear_no_bias
 from .linear import LinearNoBiasReLU as linear_fused_relu
 from .linear import MLPReLU as mlp_fused_relu
+from .linear import PackedLinearNoBias as linear_no_bias_packed
 from .softmax import Softmax

@@ -24,6 +24,9 @@ SIGNATURES = {
     "tf_gemm": (_i, [_vp, _i, _i, _i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i, _vp, _i64]),
     "tf_gemm_out": (_i, [_vp, _i, _i, _i, _i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i, _vp, _i64,
                          _vp, _i64]),
+    "tf_gemm_out_chunked": (_i, [_vp, _i, _i, _i, _i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _i64, _i64,
+                                 _vp, _i, _vp, _i64, _vp, _i64]),
+    "tf_cast_pack": (_i, [_vp, _i, _i, _i, _i64, _i64, _vp, _i64, _vp, _i64]),
     "tf_gemm_workspace_bytes": (_i64, [_i, _i, _i64, _i64, _i64]),
     "tf_gemm_tune": (_i, [_i, _i]),
     "tf_gemm_debug_flags": (_i, [_i]),

@@ -44,7 +44,16 @@ struct GemmParams {
   int out_f32;  // C holds fp32 instead of T
   const void* mask;  // optional (M, N) activation of type T: C = mask > 0 ? C : 0
   int64_t ldmask;
+  // Output split into column blocks of chunk_n columns, each its own (M, chunk_n) matrix
+  // with leading dimension ldc, chunk_skip + chunk_n elements after the previous one.
+  // One matrix: chunk_n = N, chunk_skip = 0.
+  int chunk_n;
+  int64_t chunk_skip;
 };
+
+__device__ __forceinline__ int64_t c_index(const GemmParams& p, int m, int n) {
+  return (int64_t)m * p.ldc + n + (int64_t)(n / p.chunk_n) * p.chunk_skip;
+}
 
 // ---------------------------------------------------------------------------
 // One operand panel: R rows (m or n) by BK of the contraction.
@@ -165,7 +174,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
               if (n + e < p.N && !((float)mk[e] > 0.f)) v[e] = 0.f;  // no bias / ReLU with a mask (host check)
           }
           if (p.out_f32) {
-            float* Cf = reinterpret_cast<float*>(p.C) + (int64_t)m * p.ldc + n;
+            float* Cf = reinterpret_cast<float*>(p.C) + c_index(p, m, n);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               if (n + e < p.N) {
@@ -182,13 +191,13 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
             }
 #pragma unroll
             for (int e = 0; e < 4; ++e) o[e] = (T)(p.relu ? fmaxf(v[e], 0.f) : v[e]);
-            *reinterpret_cast<typename Vec<T>::v4*>(C + (int64_t)m * p.ldc + n) = o;
+            *reinterpret_cast<typename Vec<T>::v4*>(C + c_index(p, m, n)) = o;
           } else {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               if (n + e < p.N) {
                 float x = v[e] + (bias ? (float)bias[n + e] : 0.f);
-                C[(int64_t)m * p.ldc + n + e] = (T)(p.relu ? fmaxf(x, 0.f) : x);
+                C[c_index(p, m, n) + e] = (T)(p.relu ? fmaxf(x, 0.f) : x);
               }
             }
           }
@@ -466,7 +475,7 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x16 (&
             val = __builtin_bit_cast(u32x4, cv);
           }
         }
-        st16(C + (int64_t)m * p.ldc + n, val);
+        st16(C + c_index(p, m, n), val);
       }
     }
   }
@@ -614,7 +623,7 @@ __global__ __launch_bounds__(WM* WN * 64, WPE) void gemm_dma_kernel(GemmParams p
 template <typename T, typename TO, bool VEC4>
 __global__ __launch_bounds__(256) void gemm_reduce(int M, int N, int splits, const float* __restrict__ partial,
                                                     const T* __restrict__ bias, int relu, TO* __restrict__ C,
-                                                    int64_t ldc) {
+                                                    int64_t ldc, int chunk_n, int64_t chunk_skip) {
   const int64_t total = (int64_t)M * N;
   if (VEC4) {
     const int64_t quads = total >> 2;
@@ -633,7 +642,7 @@ __global__ __launch_bounds__(256) void gemm_reduce(int M, int N, int splits, con
       Quad qd;
 #pragma unroll
       for (int e = 0; e < 4; ++e) qd.v[e] = o[e];
-      *reinterpret_cast<Quad*>(C + (int64_t)m * ldc + n) = qd;
+      *reinterpret_cast<Quad*>(C + (int64_t)m * ldc + n + (int64_t)(n / chunk_n) * chunk_skip) = qd;
     }
   } else {
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
@@ -641,7 +650,7 @@ __global__ __launch_bounds__(256) void gemm_reduce(int M, int N, int splits, con
       for (int k = 0; k < splits; ++k) s += partial[(int64_t)k * total + i];
       const int m = (int)(i / N), n = (int)(i - (int64_t)m * N);
       if (bias) s += (float)bias[n];
-      C[(int64_t)m * ldc + n] = (TO)(relu ? fmaxf(s, 0.f) : s);
+      C[(int64_t)m * ldc + n + (int64_t)(n / chunk_n) * chunk_skip] = (TO)(relu ? fmaxf(s, 0.f) : s);
     }
   }
 }
@@ -808,14 +817,16 @@ static int gemm_dispatch(hipStream_t st, int la, int lb, bool vec, const GemmPla
   if (rc != TF_OK) return rc;
   if (p.splits > 1) {
     const int64_t total = (int64_t)p.M * p.N;
-    const bool v4 = p.N % 4 == 0 && p.ldc % 4 == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0;
+    const bool v4 = p.N % 4 == 0 && p.ldc % 4 == 0 && p.chunk_n % 4 == 0 && p.chunk_skip % 4 == 0 &&
+                    (reinterpret_cast<uintptr_t>(p.C) & 15) == 0;
     int64_t blocks = ((v4 ? total / 4 : total) + 255) / 256;
     if (blocks > 4096) blocks = 4096;
     if (blocks < 1) blocks = 1;
     const dim3 g((unsigned)blocks), b(256);
     const T* bias = (const T*)p.bias;
 #define REDUCE(TO, V4) \
-  gemm_reduce<T, TO, V4><<<g, b, 0, st>>>(p.M, p.N, p.splits, p.partial, bias, p.relu, (TO*)p.C, p.ldc)
+  gemm_reduce<T, TO, V4><<<g, b, 0, st>>>(p.M, p.N, p.splits, p.partial, bias, p.relu, (TO*)p.C, p.ldc, p.chunk_n, \
+                                          p.chunk_skip)
     if (p.out_f32) { if (v4) REDUCE(float, true); else REDUCE(float, false); }
     else { if (v4) REDUCE(T, true); else REDUCE(T, false); }
 #undef REDUCE
@@ -868,16 +879,29 @@ extern "C" int tf_gemm_out(void* stream, int dtype, int out_dtype, int layout_a,
                            int64_t K, const void* A, int64_t lda, const void* B, int64_t ldb, void* C, int64_t ldc,
                            const void* bias, int relu, const void* mask_act, int64_t ld_mask, void* workspace,
                            int64_t workspace_bytes) {
+  return tf_gemm_out_chunked(stream, dtype, out_dtype, layout_a, layout_b, M, N, K, A, lda, B, ldb, C, ldc, 0, 0, bias,
+                             relu, mask_act, ld_mask, workspace, workspace_bytes);
+}
+
+extern "C" int tf_gemm_out_chunked(void* stream, int dtype, int out_dtype, int layout_a, int layout_b, int64_t M,
+                                   int64_t N, int64_t K, const void* A, int64_t lda, const void* B, int64_t ldb,
+                                   void* C, int64_t ldc, int64_t chunk_n, int64_t chunk_stride, const void* bias,
+                                   int relu, const void* mask_act, int64_t ld_mask, void* workspace,
+                                   int64_t workspace_bytes) {
   if (!A || !B || !C) return TF_EINVAL;
+  if (chunk_n < 0 || chunk_stride < 0) return TF_EINVAL;
   if (mask_act && (bias || relu || ld_mask < N)) return TF_EINVAL;
   if (out_dtype != dtype && out_dtype != TF_F32) return TF_EDTYPE;
   if (M <= 0 || N <= 0 || K <= 0 || M > 0x7fffff00 || N > 0x7fffff00 || K > 0x7fffff00) return TF_EINVAL;
+  if (chunk_n == 0 || chunk_n >= N) { chunk_n = N; chunk_stride = N; }
+  else if (N % chunk_n != 0 || chunk_n % 8 != 0 || chunk_stride % 8 != 0 ||
+           chunk_stride < (M - 1) * ldc + chunk_n) return TF_ESHAPE;
   if ((layout_a != TF_OP_KMAJOR && layout_a != TF_OP_KMINOR) || (layout_b != TF_OP_KMAJOR && layout_b != TF_OP_KMINOR))
     return TF_EINVAL;
   if (dtype != TF_F16 && dtype != TF_BF16) return TF_EDTYPE;
   const int64_t a_contig = layout_a == TF_OP_KMAJOR ? K : M;
   const int64_t b_contig = layout_b == TF_OP_KMAJOR ? K : N;
-  if (lda < a_contig || ldb < b_contig || ldc < N) return TF_ESHAPE;
+  if (lda < a_contig || ldb < b_contig || ldc < chunk_n) return TF_ESHAPE;
   if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B) | reinterpret_cast<uintptr_t>(C) |
        reinterpret_cast<uintptr_t>(bias)) & 1)
     return TF_EALIGN;
@@ -902,6 +926,8 @@ extern "C" int tf_gemm_out(void* stream, int dtype, int out_dtype, int layout_a,
   p.out_f32 = out_dtype == TF_F32 ? 1 : 0;
   p.mask = mask_act;
   p.ldmask = ld_mask;
+  p.chunk_n = (int)chunk_n;
+  p.chunk_skip = chunk_stride - chunk_n;
   hipStream_t st = (hipStream_t)stream;
   if (dtype == TF_F16) return gemm_dispatch<f16>(st, layout_a, layout_b, vec, pl, p);
   return gemm_dispatch<bf16>(st, layout_a, layout_b, vec, pl, p);

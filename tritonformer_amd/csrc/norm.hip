@@ -8,17 +8,6 @@ namespace tfa {
 
 constexpr int kRowsPerBlock = 4;  // 4 waves per workgroup, one row each
 
-// 8 consecutive affine parameters as fp32; TP = the 16-bit activation type or float
-// (fp32 master parameters are read as they are, no 16-bit copy is made first).
-template <typename TP> __device__ __forceinline__ void load8(const TP* p, float (&v)[8]) { Chunk<TP>::load(p, v); }
-template <> __device__ __forceinline__ void load8<float>(const float* p, float (&v)[8]) {
-  float a[4], b[4];
-  Chunk<float>::load(p, a);
-  Chunk<float>::load(p + 4, b);
-#pragma unroll
-  for (int i = 0; i < 4; ++i) { v[i] = a[i]; v[4 + i] = b[i]; }
-}
-
 // ---------------------------------------------------------------------------
 // LayerNorm forward.  NV = 16-byte chunks per lane (row length <= NV*64*8).
 // ---------------------------------------------------------------------------

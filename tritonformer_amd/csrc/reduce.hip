@@ -131,6 +131,48 @@ static int relu_mask_launch(hipStream_t st, int64_t rows, int64_t cols, const vo
   return TF_OK;
 }
 
+// ---------------------------------------------------------------------------
+// Convert up to four (rows, cols) matrices to 16 bits, side by side in one matrix.
+// ---------------------------------------------------------------------------
+struct PackSources { const void* p[4]; };
+
+template <typename TI, typename TO, bool VEC>
+__global__ __launch_bounds__(256) void cast_pack(PackSources src, int count, int64_t rows, int cols, int64_t ld_src,
+                                                  TO* __restrict__ dst, int64_t ld_dst) {
+  const int per_row = VEC ? cols >> 3 : cols;  // work items per source row
+  const int64_t total = rows * count * per_row;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int c = (int)(i % per_row);
+    const int64_t rj = i / per_row;
+    const int j = (int)(rj % count);
+    const int64_t r = rj / count;
+    const TI* s = (const TI*)src.p[j] + r * ld_src;
+    TO* d = dst + r * ld_dst + (int64_t)j * cols;
+    if (VEC) {
+      float v[8];
+      load8<TI>(s + c * 8, v);
+      Chunk<TO>::store(d + c * 8, v);
+    } else {
+      d[c] = (TO)(float)s[c];
+    }
+  }
+}
+
+template <typename TI, typename TO>
+static int cast_pack_launch(hipStream_t st, int count, int64_t rows, int64_t cols, const void* const* srcs,
+                            int64_t ld_src, void* dst, int64_t ld_dst) {
+  PackSources ps = {};
+  bool vec = cols % 8 == 0 && ld_src % 8 == 0 && ld_dst % 8 == 0 && aligned16(dst);
+  for (int j = 0; j < count; ++j) { ps.p[j] = srcs[j]; vec = vec && aligned16(srcs[j]); }
+  const int64_t items = rows * count * (vec ? cols / 8 : cols);
+  int64_t blocks = (items + 255) / 256;
+  if (blocks > 8192) blocks = 8192;
+  if (vec) cast_pack<TI, TO, true><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(ps, count, rows, (int)cols, ld_src, (TO*)dst, ld_dst);
+  else cast_pack<TI, TO, false><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(ps, count, rows, (int)cols, ld_src, (TO*)dst, ld_dst);
+  TF_CHECK_LAUNCH();
+  return TF_OK;
+}
+
 }  // namespace tfa
 
 using namespace tfa;
@@ -160,4 +202,21 @@ extern "C" int tf_relu_mask(void* stream, int dtype, int64_t rows, int64_t cols,
   if (dtype == TF_F16) return relu_mask_launch<f16>(st, rows, cols, grad, ldg, act, lda, out, ldo);
   if (dtype == TF_BF16) return relu_mask_launch<bf16>(st, rows, cols, grad, ldg, act, lda, out, ldo);
   return TF_EDTYPE;
+}
+
+extern "C" int tf_cast_pack(void* stream, int src_dtype, int dst_dtype, int count, int64_t rows, int64_t cols,
+                            const void* const* srcs, int64_t ld_src, void* dst, int64_t ld_dst) {
+  if (!srcs || !dst || count < 1 || count > 4) return TF_EINVAL;
+  for (int j = 0; j < count; ++j)
+    if (!srcs[j]) return TF_EINVAL;
+  if (rows < 0 || cols <= 0 || cols > (1 << 30) || ld_src < cols || ld_dst < count * cols) return TF_EINVAL;
+  if (dst_dtype != TF_F16 && dst_dtype != TF_BF16) return TF_EDTYPE;
+  if (src_dtype != TF_F32 && src_dtype != dst_dtype) return TF_EDTYPE;
+  if (rows == 0) return TF_OK;
+  hipStream_t st = (hipStream_t)stream;
+  if (dst_dtype == TF_F16)
+    return src_dtype == TF_F32 ? cast_pack_launch<float, f16>(st, count, rows, cols, srcs, ld_src, dst, ld_dst)
+                               : cast_pack_launch<f16, f16>(st, count, rows, cols, srcs, ld_src, dst, ld_dst);
+  return src_dtype == TF_F32 ? cast_pack_launch<float, bf16>(st, count, rows, cols, srcs, ld_src, dst, ld_dst)
+                             : cast_pack_launch<bf16, bf16>(st, count, rows, cols, srcs, ld_src, dst, ld_dst);
 }

@@ -25,6 +25,17 @@ template <> struct Chunk<float> {
   }
 };
 
+// 8 consecutive elements as fp32; TP = a 16-bit type or float (fp32 master parameters are
+// read as they are, no 16-bit copy is made first).
+template <typename TP> __device__ __forceinline__ void load8(const TP* p, float (&v)[8]) { Chunk<TP>::load(p, v); }
+template <> __device__ __forceinline__ void load8<float>(const float* p, float (&v)[8]) {
+  float a[4], b[4];
+  Chunk<float>::load(p, a);
+  Chunk<float>::load(p + 4, b);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { v[i] = a[i]; v[4 + i] = b[i]; }
+}
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 // True when rows of `n` elements of T starting at p with leading dimension ld

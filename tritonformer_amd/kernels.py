@@ -7,6 +7,7 @@ They take the place of the launchers under the reference's
 scratch buffers are ``torch.empty`` tensors owned by the caller's allocator;
 the native side keeps nothing.
 """
+import ctypes
 import math
 from functools import lru_cache
 
@@ -28,14 +29,15 @@ def _gemm_ws(la, lb, m, n, k):
     return load().tf_gemm_workspace_bytes(la, lb, m, n, k)
 
 
-def _gemm(dtype, la, lb, m, n, k, a, lda, b, ldb, c, ldc, bias, relu, mask=None):
+def _gemm(dtype, la, lb, m, n, k, a, lda, b, ldb, c, ldc, bias, relu, mask=None, chunk_n=0, chunk_stride=0):
     lib = load()
     ws_bytes = 0 if mask is not None else _gemm_ws(la, lb, m, n, k)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=c.device) if ws_bytes else None
-    check(lib.tf_gemm_out(stream_ptr(), dtype_code(dtype), dtype_code(c.dtype), la, lb, m, n, k, a.data_ptr(), lda,
-                          b.data_ptr(), ldb, c.data_ptr(), ldc, bias.data_ptr() if bias is not None else None,
-                          int(relu), mask.data_ptr() if mask is not None else None, n if mask is not None else 0,
-                          ws.data_ptr() if ws is not None else None, ws_bytes))
+    check(lib.tf_gemm_out_chunked(stream_ptr(), dtype_code(dtype), dtype_code(c.dtype), la, lb, m, n, k, a.data_ptr(),
+                                  lda, b.data_ptr(), ldb, c.data_ptr(), ldc, chunk_n, chunk_stride,
+                                  bias.data_ptr() if bias is not None else None, int(relu),
+                                  mask.data_ptr() if mask is not None else None, n if mask is not None else 0,
+                                  ws.data_ptr() if ws is not None else None, ws_bytes))
 
 
 def _check_linear(a, b, bias=None):
@@ -87,12 +89,14 @@ def mm(a, b, fuse_relu=False, mask_act=None):
     return gemm(a, b, None, fuse_relu, mask_act)
 
 
-def mm_dw(x, grad, out_dtype=None):
+def mm_dw(x, grad, out_dtype=None, chunks=1):
     """``sum_b x[b]^T @ grad[b]`` -> (in, out): reference ``bmm`` of the
     transposed view (kernels/gemm.py:161-200) followed by ``torch.sum`` over the
     batch (linear.py:24-25), as ONE contraction over all B*S tokens.
     ``out_dtype=torch.float32`` stores the fp32 accumulators unrounded (gradient
-    of an fp32 master weight)."""
+    of an fp32 master weight).  ``chunks=c > 1`` returns (c, in, out/c): the
+    column blocks of the product as c separate contiguous matrices (the gradients
+    of c weights whose outputs were computed side by side in one product)."""
     if x.shape[:-1] != grad.shape[:-1]:
         raise ValueError("Leading dimensions of the two operands do not match")
     if x.dtype != grad.dtype:
@@ -100,8 +104,34 @@ def mm_dw(x, grad, out_dtype=None):
     require_cuda(x, grad)
     x2, t, kin = _rows2d(x)
     g2, _, nout = _rows2d(grad)
+    if chunks > 1:
+        if nout % chunks or (nout // chunks) % 8:
+            raise ValueError("column blocks must be equal and multiples of 8 wide")
+        each = nout // chunks
+        out = torch.empty((chunks, kin, each), dtype=out_dtype or x.dtype, device=x.device)
+        _gemm(x.dtype, KMINOR, KMINOR, kin, nout, t, x2, kin, g2, nout, out, each, None, False,
+              chunk_n=each, chunk_stride=kin * each)
+        return out
     out = torch.empty((kin, nout), dtype=out_dtype or x.dtype, device=x.device)
     _gemm(x.dtype, KMINOR, KMINOR, kin, nout, t, x2, kin, g2, nout, out, nout, None, False)
+    return out
+
+
+def cast_pack(weights, dtype):
+    """The (in, out_j) matrices ``weights`` (all one shape and dtype: float32 or ``dtype``)
+    converted to the 16-bit ``dtype`` side by side in one (in, sum out_j) matrix, one launch."""
+    w0 = weights[0]
+    if not 1 <= len(weights) <= 4 or any(w.shape != w0.shape or w.dtype != w0.dtype or w.ndim != 2 for w in weights):
+        raise ValueError("cast_pack takes 1..4 matrices of one shape and dtype")
+    if dtype not in (torch.float16, torch.bfloat16) or w0.dtype not in (torch.float32, dtype):
+        raise TypeError("cast_pack converts float32 (or already 16-bit) matrices to float16 / bfloat16")
+    require_cuda(*weights)
+    weights = [w if w.is_contiguous() else w.contiguous() for w in weights]
+    rows, cols = w0.shape
+    out = torch.empty((rows, len(weights) * cols), dtype=dtype, device=w0.device)
+    ptrs = (ctypes.c_void_p * len(weights))(*[w.data_ptr() for w in weights])
+    check(load().tf_cast_pack(stream_ptr(), dtype_code(w0.dtype), dtype_code(dtype), len(weights), rows, cols, ptrs,
+                              cols, out.data_ptr(), len(weights) * cols))
     return out
 
 

@@ -4,7 +4,7 @@ import torch
 from torch.autograd import Function
 
 from ._amp import amp_bwd, amp_fwd
-from .kernels import gemm, mask_grad, mm, mm_dw, unbroadcast_leading
+from .kernels import cast_pack, gemm, mask_grad, mm, mm_dw, unbroadcast_leading
 
 
 def _grads(ctx, grad_output, inputs, weights):
@@ -123,3 +123,30 @@ class MLPReLU(Function):
         grad_w1 = mm_dw(input, grad_hidden, out_dtype=f32 if ctx.arg_dtypes[1] == f32 else None)
         grad_b1 = unbroadcast_leading(grad_hidden) if ctx.has_bias[0] else None
         return grad_input, grad_w1, grad_b1, grad_w2, grad_b2
+
+
+class PackedLinearNoBias(Function):
+    """``apply(x, W_0, ..., W_{c-1})`` (c <= 4 weights of one shape (in, out)) returns
+    x @ [W_0 | ... | W_{c-1}], shape (B, S, c*out): c bias-free projections of the same
+    input (the q, k, v projections of reference transformer.py:158-160) as ONE product.
+    The 16-bit side-by-side operand is built from the weights as they are stored (fp32
+    master weights under autocast, or 16-bit) by one conversion kernel; the backward is
+    one dX product and one dW product whose column blocks land in c separate contiguous
+    gradients.  Same arithmetic per output element as c LinearNoBias calls."""
+
+    @staticmethod
+    @amp_fwd(keep=(1, 2, 3, 4))
+    def forward(ctx, input, *weights):
+        packed = cast_pack(weights, input.dtype)
+        ctx.save_for_backward(input, packed)
+        ctx.count = len(weights)
+        ctx.weight_dtype = weights[0].dtype
+        return mm(input, packed)
+
+    @staticmethod
+    @amp_bwd
+    def backward(ctx, grad_output):
+        input, packed = ctx.saved_tensors
+        grad_input = mm(grad_output, packed.T) if ctx.needs_input_grad[0] else None
+        grad_w = mm_dw(input, grad_output, out_dtype=ctx.weight_dtype, chunks=ctx.count)
+        return (grad_input,) + tuple(grad_w[j] for j in range(ctx.count))

@@ -23,7 +23,7 @@ from . import (
     fast_causal_attention,
     fast_causal_attention_qkvpacked,
     fast_causal_attention_with_bias,
-    linear_no_bias,
+    linear_no_bias_packed,
     mlp_fused_relu,
     shifted_cross_entropy_loss,
 )
@@ -127,10 +127,10 @@ class CausalAttention(nn.Module):
     def forward(self, hidden_states: torch.Tensor, attn_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
         batch_size, q_seq_len, hidden_dim = hidden_states.shape
         if FUSE_QKV:
-            # one (d, 3d) GEMM instead of three (d, d): same parameters, concatenated on the fly;
-            # autograd splits the weight gradient back into the three parameters
-            w_qkv = torch.cat([self.q_proj.weight, self.k_proj.weight, self.v_proj.weight], dim=1)
-            qkv = linear_no_bias.apply(hidden_states, w_qkv)
+            # one (d, 3d) GEMM instead of three (d, d): same parameters, laid side by side in
+            # 16 bits by one conversion kernel; the weight gradient comes back as three tensors
+            qkv = linear_no_bias_packed.apply(hidden_states, self.q_proj.weight, self.k_proj.weight,
+                                              self.v_proj.weight)
             qkv = qkv.view(batch_size, q_seq_len, 3, self.num_attention_heads, self.hidden_size_per_attention_head)
             return self.out_proj(fast_causal_attention_qkvpacked.apply(qkv, attn_bias))
         query_layer = self._heads(self.q_proj(hidden_states))
