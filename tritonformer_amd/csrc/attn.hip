@@ -21,8 +21,9 @@
 #include <type_traits>
 #include "rowops.h"
 
-
 namespace tfa {
+
+typedef __attribute__((address_space(1))) const void gptr_void;
 
 struct AttnParams {
   const void *q, *k, *v, *o, *d_o;
@@ -103,6 +104,16 @@ template <typename T> __device__ __forceinline__ typename Vec<T>::v8 round8(cons
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// max(x, x of lane l ^ 32) through the VALU (v_permlane32_swap) rather than the LDS crossbar:
+// swapping the upper half of one copy of x with the lower half of another leaves, in every
+// lane, its own value in one register and its partner's in the other.
+__device__ __forceinline__ float max_with_other_half(float x) {
+  const unsigned u = __builtin_bit_cast(unsigned, x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  const unsigned r0 = r[0], r1 = r[1];
+  return fmaxf(__builtin_bit_cast(float, r0), __builtin_bit_cast(float, r1));
+}
+
 // Register r of a 32x32 MFMA result covers row (r/4)*8 + 4*(lane/32) + r%4.
 __device__ __forceinline__ int reg_row(int r, int lane) { return (r >> 2) * 8 + 4 * (lane >> 5) + (r & 3); }
 
@@ -122,12 +133,13 @@ __device__ __forceinline__ int reg_row(int r, int lane) { return (r >> 2) * 8 + 
 constexpr float kRescaleThreshold = 8.0f;  // log2 domain
 
 template <typename T, int HD, bool HAS_BIAS>
-__global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_fwd_kernel(AttnParams p) {
+__global__ __launch_bounds__(256, HD > 64 ? 1 : 3) void attn_fwd_kernel(AttnParams p) {
   typedef SeqTile<T, 64, HD> KT;
   typedef typename Vec<T>::v8 v8;
   typedef typename Vec<T>::v4 v4;
   constexpr int KS = HD / 16, DT = HD / 32;
   constexpr int STAGE = 2 * KT::BYTES;
+  constexpr int PT = KT::PER_THREAD;  // 16-byte chunks per thread per 64-row tile
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -170,38 +182,72 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_fw
     for (int r = 0; r < 16; ++r) oacc[d][r] = 0.f;
   float m_ref = -INFINITY;  // reference maximum (log2 domain) the accumulators are scaled to
 
-  u32x4 rk[KT::PER_THREAD], rv[KT::PER_THREAD];
-  KT::fetch(rk, K, p.ss, 0);
-  KT::fetch(rv, V, p.ss, 0);
-  KT::commit(smem, rk);
-  KT::commit(smem + KT::BYTES, rv);
+  // K and V tiles go from global memory straight into LDS (no register staging): thread
+  // t's j-th 16-byte load lands in LDS slot t + 256 j of the tile, so the chunk swizzle of
+  // the tile layout is applied to the global address instead.
+  const T* kp[PT];
+#pragma unroll
+  for (int j = 0; j < PT; ++j) {
+    const int id = threadIdx.x + j * 256;
+    const int row = id / KT::CPR, c = (id % KT::CPR) ^ KT::swz(row);
+    kp[j] = K + (int64_t)row * p.ss + c * 8;
+  }
+  const int64_t v_minus_k = V - K;
+  auto load_tile = [&](int stage_off) {  // next 64 keys / values into the stage at byte offset stage_off
+#pragma unroll
+    for (int j = 0; j < PT; ++j) {
+      char* dst = smem + stage_off + (j * 256 + wave * 64) * 16;
+      __builtin_amdgcn_global_load_lds((gptr_void*)kp[j], (lds_void*)dst, 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_void*)(kp[j] + v_minus_k), (lds_void*)(dst + KT::BYTES), 16, 0, 0);
+      kp[j] += (int64_t)64 * p.ss;
+    }
+  };
+  // lane-dependent parts of the LDS operand addresses; block, sub-tile and stage offsets are
+  // compile-time constants that end up in the instructions' offset fields
+  uint32_t ka[KS], va[DT][2];
+  const uint32_t lds0 = lds_address(smem);
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) ka[ks] = lds0 + KT::addr(lane & 31, ks * 2 + (lane >> 5));
+#pragma unroll
+  for (int d = 0; d < DT; ++d) {
+    const int i = lane & 15;
+    const int col = d * 32 + 16 * ((lane >> 4) & 1) + (i & 3) * 4;
+    const int r0 = 4 * (lane >> 5) + (i >> 2);
+    va[d][0] = lds0 + KT::addr(r0, col >> 3) + (col & 7) * 2;
+    va[d][1] = lds0 + KT::addr(r0 + 8, col >> 3) + (col & 7) * 2;
+  }
+
+  load_tile(0);
   __syncthreads();
 
-  for (int j = 0; j < nkv; ++j) {
-    const char* sk = smem + (j & 1) * STAGE;
-    const char* sv = sk + KT::BYTES;
-    const bool more = j + 1 < nkv;
-    if (more) {
-      KT::fetch(rk, K, p.ss, (j + 1) * 64);
-      KT::fetch(rv, V, p.ss, (j + 1) * 64);
-    }
+  // One 64-key block out of the stage at byte offset SOFF.
+  auto step = [&](auto stage_tag, int j) {
+    constexpr int SOFF = decltype(stage_tag)::value * STAGE;
+    constexpr int VOFF = SOFF + KT::BYTES;
+    if (j + 1 < nkv) load_tile(STAGE - SOFF);
     const int kb = j * 64;
     if (active && kb <= q0w + 31) {
       auto block = [&](auto diag_tag) {
         constexpr bool DIAG = decltype(diag_tag)::value;
         // on a diagonal block the second 32-key half may lie entirely above the diagonal
         const bool live1 = !DIAG || kb + 32 <= q0w + 31;
+        // all K operands of the block are requested before the first MFMA
+        u32x4 kf[2][KS];
+        static_for<2 * KS>([&](auto it) {
+          constexpr int jt = decltype(it)::value % 2, ks = decltype(it)::value / 2;  // the two halves alternate
+          lds_read128_at<SOFF + jt * 32 * HD * 2>(kf[jt][ks], ka[ks]);
+        });
         f32x16 st[2];
 #pragma unroll
-        for (int jt = 0; jt < 2; ++jt) {
+        for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
           for (int r = 0; r < 16; ++r) st[jt][r] = 0.f;
-          if (jt == 0 || live1) {
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) st[jt] = mfma32(KT::frag_rows(sk, jt * 32, ks, lane), qf[ks], st[jt]);
-          }
-        }
-        // x = s * scale * log2e (+ bias * log2e), masked; block maximum
+        static_for<2 * KS>([&](auto it) {
+          constexpr int idx = decltype(it)::value, jt = idx % 2, ks = idx / 2;  // two independent accumulation chains
+          lds_wait<2 * KS - 1 - idx>(kf[jt][ks]);
+          st[jt] = mfma32(__builtin_bit_cast(v8, kf[jt][ks]), qf[ks], st[jt]);
+        });
+        // block maximum; without bias it is taken over the raw scores and scaled once
         float mx = -INFINITY;
 #pragma unroll
         for (int jt = 0; jt < 2; ++jt) {
@@ -216,14 +262,25 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_fw
             }
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-              float x = HAS_BIAS ? fmaf(st[jt][g * 4 + e], p.scale_log2, bv[e]) : st[jt][g * 4 + e] * p.scale_log2;
+              float x = st[jt][g * 4 + e];
+              if (HAS_BIAS) x = fmaf(x, p.scale_log2, bv[e]);
               if (DIAG && (key0 + e > myq || (jt == 1 && !live1))) x = -INFINITY;
               st[jt][g * 4 + e] = x;
               mx = fmaxf(mx, x);
             }
           }
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        // the V operands are requested now and arrive while the exponentials are computed
+        constexpr int NVF = 4 * DT;  // operands of the block: (32-key half, 16-key step, 32-wide hd slice)
+        u32x2 vlo[NVF], vhi[NVF];
+        static_for<NVF>([&](auto it) {
+          constexpr int idx = decltype(it)::value, jt = idx / (2 * DT), t = (idx / DT) % 2, d = idx % DT;
+          constexpr int off = VOFF + (jt * 32 + t * 16) * HD * 2;
+          lds_read64_tr_at<off>(vlo[idx], va[d][0]);
+          lds_read64_tr_at<off>(vhi[idx], va[d][1]);
+        });
+        mx = max_with_other_half(mx);
+        if (!HAS_BIAS) mx *= p.scale_log2;  // scale > 0: max(s) * scale = max(s * scale)
         // raise the reference maximum only when some row outgrew it by 2^8
         const bool grow = mx > m_ref + kRescaleThreshold;
         if (__any(grow)) {
@@ -241,29 +298,31 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_fw
 #pragma unroll
         for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) st[jt][r] = fast_exp2(st[jt][r] - m_use);
-#pragma unroll
-        for (int jt = 0; jt < 2; ++jt) {
-          if (jt == 0 || live1) {
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-              const v8 pb = round8<T>(st[jt], t);
-              lacc = mfma32(ones, pb, lacc);  // every row of lacc = sum over keys of P
-#pragma unroll
-              for (int d = 0; d < DT; ++d) oacc[d] = mfma32(KT::frag_hd(sv, jt * 32 + t * 16, d, lane), pb, oacc[d]);
-            }
-          }
-        }
+          for (int r = 0; r < 16; ++r)
+            st[jt][r] = fast_exp2(HAS_BIAS ? st[jt][r] - m_use : fmaf(st[jt][r], p.scale_log2, -m_use));
+        // every requested operand is consumed (a half above the diagonal contributes P = 0)
+        static_for<4>([&](auto it) {
+          constexpr int jt = decltype(it)::value / 2, t = decltype(it)::value % 2;
+          const v8 pb = round8<T>(st[jt], t);
+          lacc = mfma32(ones, pb, lacc);  // every row of lacc = sum over keys of P
+          static_for<DT>([&](auto dd) {
+            constexpr int d = decltype(dd)::value, idx = (jt * 2 + t) * DT + d;
+            constexpr int later = 2 * (NVF - 1 - idx);  // LDS reads requested after this operand
+            lds_wait<(later < 15 ? later : 15)>(vhi[idx]);
+            const u32x4 v = {vlo[idx][0], vlo[idx][1], vhi[idx][0], vhi[idx][1]};
+            oacc[d] = mfma32(__builtin_bit_cast(v8, v), pb, oacc[d]);
+          });
+        });
       };
       if (kb + 63 > q0w) block(std::true_type{});
       else block(std::false_type{});
     }
-    if (more) {
-      char* dk = smem + ((j + 1) & 1) * STAGE;
-      KT::commit(dk, rk);
-      KT::commit(dk + KT::BYTES, rv);
-    }
-    __syncthreads();
+    __syncthreads();  // waits for this thread's tile loads, then for everyone's; all reads of this stage are done
+  };
+
+  for (int j = 0; j < nkv; j += 2) {
+    step(std::integral_constant<int, 0>{}, j);
+    if (j + 1 < nkv) step(std::integral_constant<int, 1>{}, j + 1);
   }
 
   if (active) {

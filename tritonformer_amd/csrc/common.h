@@ -1,6 +1,8 @@
 // Shared device helpers for the gfx950 kernels: 16-bit types, 16-byte vector
 // access, wave64 reductions and MFMA wrappers.  gfx950 only, wave size 64.
 #pragma once
+#include <type_traits>
+#include <utility>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include "../../include/tritonformer_amd.h"
@@ -85,6 +87,42 @@ __device__ __forceinline__ u32x2 lds_ld8_tr(const char* base, int byte_off) {
   typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
   s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(base + byte_off));
   return __builtin_bit_cast(u32x2, v);
+}
+
+// ---- LDS reads as volatile asm ---------------------------------------------
+// The compiler neither reorders these nor waits for them (and does not make them
+// wait for direct-to-LDS global loads it cannot tell apart), so a kernel decides
+// how far ahead of their consumers they run.  Every consumer must sit behind
+// lds_wait<N>(reg): it waits until at most N later LDS operations are outstanding
+// and is tied to the register, so the consumer cannot be scheduled above it.
+// A register that was requested must always be waited for before it dies.
+__device__ __forceinline__ uint32_t lds_address(const char* p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
+}
+template <int OFF> __device__ __forceinline__ void lds_read128_at(u32x4& dst, uint32_t addr) {
+  static_assert(OFF >= 0 && OFF < 65536, "offset field is 16 bits");
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+template <int OFF> __device__ __forceinline__ void lds_read64_tr_at(u32x2& dst, uint32_t addr) {
+  static_assert(OFF >= 0 && OFF < 65536, "offset field is 16 bits");
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+template <int N, typename R> __device__ __forceinline__ void lds_wait(R& reg) {
+  static_assert(N >= 0 && N <= 15, "lgkmcnt is 4 bits");
+  asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(reg) : "n"(N));
+}
+
+// s_waitcnt vmcnt(n) with the other counters unconstrained (gfx9 encoding).
+template <int N> __device__ __forceinline__ void wait_vmcnt() {
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+// f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N-1>{})
+template <typename F, int... I> __device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F> __device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
 inline int ceil_div(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }

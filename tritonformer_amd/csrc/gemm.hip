@@ -312,9 +312,6 @@ template <int N> __device__ __forceinline__ void wait_lgkmcnt() {
 // LDS operand reads issued as volatile asm: the compiler neither reorders them nor
 // waits for them, so the kernel decides how far ahead of their MFMAs they run
 // (every consumer sits behind an explicit wait_lgkmcnt + scheduling barrier).
-__device__ __forceinline__ uint32_t lds_address(const char* p) {
-  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
-}
 template <bool KMAJOR> struct FragRegs;
 template <> struct FragRegs<true> {
   u32x4 q;
@@ -400,10 +397,6 @@ struct DmaPanel {
   }
 };
 
-// s_waitcnt vmcnt(n) with the other counters unconstrained (gfx9 encoding).
-template <int N> __device__ __forceinline__ void wait_vmcnt() {
-  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
-}
 // Epilogue of the direct-to-LDS kernel.  Each wave rounds its accumulators (after
 // bias / ReLU), parks one 32-row block at a time in a private LDS region and
 // reads it back row-contiguously, so every global store instruction writes whole
