@@ -74,7 +74,7 @@ def run_steps(model, tokens, n, dtype):
 
 
 class GemmTimer:
-    """HIP events on the current (launch) stream around every tf_gemm call."""
+    """HIP events on the current (launch) stream around every tf_gemm / tf_gemm_group call."""
 
     def __init__(self):
         self.records = []
@@ -93,11 +93,24 @@ class GemmTimer:
             e1.record()
             self.records.append(((la, lb, m, n, k), e0, e1))
 
+        self._orig_group = kernels._gemm_group
+
+        def timed_group(dtype, out_dtype, la, lb, problems, device):
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record()
+            self._orig_group(dtype, out_dtype, la, lb, problems, device)
+            e1.record()
+            key = ("group",) + tuple((q.M, q.N, q.K) for q in problems)
+            self.records.append((key, e0, e1))
+
         kernels._gemm = timed
+        kernels._gemm_group = timed_group
         return self
 
     def __exit__(self, *exc):
         self._kernels._gemm = self._orig
+        self._kernels._gemm_group = self._orig_group
         torch.cuda.synchronize()
         self.by_shape = {}
         for key, e0, e1 in self.records:
@@ -220,7 +233,7 @@ def main():
             "flop_per_launch": round(gflops / launches, 1),
             "avg_launch_us": round(total_ms / launches * 1e3, 2),
             "gemm_ms_per_step": round(total_ms / reps, 3),
-            "measured": f"HIP events on the launch stream around each tf_gemm call, {reps} instrumented steps "
+            "measured": f"HIP events on the launch stream around each tf_gemm / tf_gemm_group call, {reps} instrumented steps "
                         "run after the timed ones (split-contraction launches include their reduce kernel)",
         }
     if args.calibrate_copy:

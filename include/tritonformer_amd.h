@@ -101,6 +101,26 @@ int tf_gemm_out_chunked(void* stream, int dtype, int out_dtype, int layout_a, in
                         const void* bias, int relu, const void* mask_act, int64_t ld_mask,
                         void* workspace, int64_t workspace_bytes);
 int64_t tf_gemm_workspace_bytes(int layout_a, int layout_b, int64_t M, int64_t N, int64_t K);
+
+/* `count` (1..4) independent products of one dtype and one pair of operand layouts,
+ * no bias / ReLU / mask, each with the arguments of tf_gemm_out_chunked.  When every
+ * problem meets the fast-path preconditions and both operands are TF_OP_KMINOR (the
+ * weight-gradient form x^T . dy of tritonformer/linear.py:24-25), all of them run in
+ * ONE launch: outputs with few tiles (two MLP weights: 64 tiles each) then fill the
+ * GPU side by side, with half as many contraction slices and fp32 partials as two
+ * launches would need.  Otherwise the problems run one after the other.  The results
+ * do not depend on which of the two happens beyond the fp32 summation order. */
+typedef struct tf_gemm_problem {
+  int64_t M, N, K;
+  const void* A; int64_t lda;
+  const void* B; int64_t ldb;
+  void* C; int64_t ldc;
+  int64_t chunk_n, chunk_stride;   /* 0, 0: one output matrix */
+} tf_gemm_problem;
+int tf_gemm_group(void* stream, int dtype, int out_dtype, int layout_a, int layout_b, int count,
+                  const tf_gemm_problem* problems, void* workspace, int64_t workspace_bytes);
+int64_t tf_gemm_group_workspace_bytes(int layout_a, int layout_b, int count,
+                                      const tf_gemm_problem* problems);
 /* Diagnostic, no counterpart in the reference (whose Triton autotuner picks
  * tiles per shape, kernels/gemm.py:15-79): force tile configuration `cfg`
  * (-1 = automatic) and contraction split `splits` (0 = automatic) for all

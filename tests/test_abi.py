@@ -77,6 +77,15 @@ def test_gemm_rejects_bad_arguments():
     assert chunked(36, 64 * 32) == -4 and chunked(32, 63 * 32) == -4 and chunked(32, 64 * 32, ldc=24) == -4
     assert chunked(-1, 0) == -1
     import ctypes
+    probs = (_lib.GemmProblem * 2)(_lib.GemmProblem(1024, 4096, 8192, FAKE, 1024, FAKE, 4096, FAKE, 4096, 0, 0),
+                                   _lib.GemmProblem(4096, 1024, 8192, FAKE, 4096, FAKE, 1024, FAKE, 1024, 0, 0))
+    # two 64-tile weight gradients side by side: 2 contraction slices each instead of 4
+    assert lib.tf_gemm_group_workspace_bytes(1, 1, 2, probs) == 2 * 2 * 1024 * 4096 * 4
+    assert lib.tf_gemm_workspace_bytes(1, 1, 1024, 4096, 8192) == 4 * 1024 * 4096 * 4
+    assert lib.tf_gemm_group(None, 0, 2, 1, 1, 2, probs, None, 0) == -5
+    assert lib.tf_gemm_group(None, 0, 2, 1, 1, 5, probs, FAKE, 1 << 40) == -1
+    assert lib.tf_gemm_group(None, 2, 2, 1, 1, 2, probs, FAKE, 1 << 40) == -2
+    assert lib.tf_gemm_group(None, 0, 1, 1, 1, 2, probs, FAKE, 1 << 40) == -2
     ptrs = (ctypes.c_void_p * 3)(FAKE, FAKE, FAKE)
     assert lib.tf_cast_pack(None, 2, 0, 5, 8, 8, ptrs, 8, FAKE, 40) == -1          # more than 4 sources
     assert lib.tf_cast_pack(None, 2, 0, 3, 8, 8, ptrs, 8, FAKE, 16) == -1          # destination rows too short

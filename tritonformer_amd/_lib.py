@@ -27,6 +27,8 @@ SIGNATURES = {
     "tf_gemm_out_chunked": (_i, [_vp, _i, _i, _i, _i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _i64, _i64,
                                  _vp, _i, _vp, _i64, _vp, _i64]),
     "tf_cast_pack": (_i, [_vp, _i, _i, _i, _i64, _i64, _vp, _i64, _vp, _i64]),
+    "tf_gemm_group": (_i, [_vp, _i, _i, _i, _i, _i, _vp, _vp, _i64]),
+    "tf_gemm_group_workspace_bytes": (_i64, [_i, _i, _i, _vp]),
     "tf_gemm_workspace_bytes": (_i64, [_i, _i, _i64, _i64, _i64]),
     "tf_gemm_tune": (_i, [_i, _i]),
     "tf_gemm_debug_flags": (_i, [_i]),
@@ -50,6 +52,12 @@ SIGNATURES = {
     "tf_colsum_partial_bytes": (_i64, [_i64, _i64]),
     "tf_relu_mask": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64]),
 }
+
+class GemmProblem(ctypes.Structure):
+    """`tf_gemm_problem` of include/tritonformer_amd.h."""
+    _fields_ = [("M", _i64), ("N", _i64), ("K", _i64), ("A", _vp), ("lda", _i64), ("B", _vp), ("ldb", _i64),
+                ("C", _vp), ("ldc", _i64), ("chunk_n", _i64), ("chunk_stride", _i64)]
+
 
 _lib = None
 

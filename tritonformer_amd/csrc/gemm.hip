@@ -474,8 +474,8 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x16 (&
   }
 }
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, int WPE, bool A_KMAJOR, bool B_KMAJOR>
-__global__ __launch_bounds__(WM* WN * 64, WPE) void gemm_dma_kernel(GemmParams p) {
+template <typename T, int BM, int BN, int BK, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR>
+__device__ __forceinline__ void gemm_dma_body(const GemmParams& p, const int pid) {
   constexpr int NW = WM * WN;
   constexpr int WTM = BM / WM, WTN = BN / WN;
   constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -496,7 +496,6 @@ __global__ __launch_bounds__(WM* WN * 64, WPE) void gemm_dma_kernel(GemmParams p
   const int wm = wave / WN, wn = wave % WN;
 
   const int tiles = p.tiles_m * p.tiles_n;
-  const int pid = (p.flags & 1) ? (int)blockIdx.x : remap_xcd(blockIdx.x, tiles * p.splits);
   const int split = pid / tiles;
   const int t = pid - split * tiles;
   const int per_group = GROUP_M * p.tiles_n;
@@ -609,6 +608,31 @@ __global__ __launch_bounds__(WM* WN * 64, WPE) void gemm_dma_kernel(GemmParams p
     if (p.out_f32) gemm_epilogue_lds<T, float, TM, TN, WTM, WTN>(p, acc, smem, m0, n0, wm, wn, wave, lane);
     else gemm_epilogue_lds<T, T, TM, TN, WTM, WTN>(p, acc, smem, m0, n0, wm, wn, wave, lane);
   }
+}
+
+template <typename T, int BM, int BN, int BK, int WM, int WN, int WPE, bool A_KMAJOR, bool B_KMAJOR>
+__global__ __launch_bounds__(WM* WN * 64, WPE) void gemm_dma_kernel(GemmParams p) {
+  const int pid = (p.flags & 1) ? (int)blockIdx.x : remap_xcd(blockIdx.x, p.tiles_m * p.tiles_n * p.splits);
+  gemm_dma_body<T, BM, BN, BK, WM, WN, A_KMAJOR, B_KMAJOR>(p, pid);
+}
+
+// Up to four independent products of one operand layout in ONE launch: workgroup ids
+// [first[i], first[i+1]) belong to problem i.  Used for weight gradients, whose output has
+// few tiles: side by side they fill the chip with fewer, longer contraction slices.
+constexpr int kMaxGroup = 4;
+struct GemmGroup {
+  GemmParams p[kMaxGroup];
+  int first[kMaxGroup + 1];
+  int count;
+};
+template <typename T, int BM, int BN, int BK, int WM, int WN, int WPE, bool A_KMAJOR, bool B_KMAJOR>
+__global__ __launch_bounds__(WM* WN * 64, WPE) void gemm_dma_group_kernel(GemmGroup g) {
+  const int pid = remap_xcd(blockIdx.x, g.first[g.count]);
+  int i = 0;
+#pragma unroll
+  for (int k = 1; k < kMaxGroup; ++k)
+    if (k < g.count && pid >= g.first[k]) i = k;
+  gemm_dma_body<T, BM, BN, BK, WM, WN, A_KMAJOR, B_KMAJOR>(g.p[i], pid - g.first[i]);
 }
 
 // Sum the split-contraction partials in a fixed order and apply the epilogue.
@@ -797,6 +821,28 @@ static int launch_cfg(hipStream_t st, const GemmPlan& pl, const GemmParams& p) {
   return TF_EINVAL;
 }
 
+// Second pass of a split contraction (no-op when the contraction was not split).
+template <typename T>
+static int launch_reduce(hipStream_t st, const GemmParams& p) {
+  if (p.splits <= 1) return TF_OK;
+  const int64_t total = (int64_t)p.M * p.N;
+  const bool v4 = p.N % 4 == 0 && p.ldc % 4 == 0 && p.chunk_n % 4 == 0 && p.chunk_skip % 4 == 0 &&
+                  (reinterpret_cast<uintptr_t>(p.C) & 15) == 0;
+  int64_t blocks = ((v4 ? total / 4 : total) + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  if (blocks < 1) blocks = 1;
+  const dim3 g((unsigned)blocks), b(256);
+  const T* bias = (const T*)p.bias;
+#define REDUCE(TO, V4) \
+  gemm_reduce<T, TO, V4><<<g, b, 0, st>>>(p.M, p.N, p.splits, p.partial, bias, p.relu, (TO*)p.C, p.ldc, p.chunk_n, \
+                                          p.chunk_skip)
+  if (p.out_f32) { if (v4) REDUCE(float, true); else REDUCE(float, false); }
+  else { if (v4) REDUCE(T, true); else REDUCE(T, false); }
+#undef REDUCE
+  TF_CHECK_LAUNCH();
+  return TF_OK;
+}
+
 template <typename T>
 static int gemm_dispatch(hipStream_t st, int la, int lb, bool vec, const GemmPlan& pl, const GemmParams& p) {
   const bool ak = la == TF_OP_KMAJOR, bk = lb == TF_OP_KMAJOR;
@@ -808,22 +854,22 @@ static int gemm_dispatch(hipStream_t st, int la, int lb, bool vec, const GemmPla
   else GO(false, false);
 #undef GO
   if (rc != TF_OK) return rc;
-  if (p.splits > 1) {
-    const int64_t total = (int64_t)p.M * p.N;
-    const bool v4 = p.N % 4 == 0 && p.ldc % 4 == 0 && p.chunk_n % 4 == 0 && p.chunk_skip % 4 == 0 &&
-                    (reinterpret_cast<uintptr_t>(p.C) & 15) == 0;
-    int64_t blocks = ((v4 ? total / 4 : total) + 255) / 256;
-    if (blocks > 4096) blocks = 4096;
-    if (blocks < 1) blocks = 1;
-    const dim3 g((unsigned)blocks), b(256);
-    const T* bias = (const T*)p.bias;
-#define REDUCE(TO, V4) \
-  gemm_reduce<T, TO, V4><<<g, b, 0, st>>>(p.M, p.N, p.splits, p.partial, bias, p.relu, (TO*)p.C, p.ldc, p.chunk_n, \
-                                          p.chunk_skip)
-    if (p.out_f32) { if (v4) REDUCE(float, true); else REDUCE(float, false); }
-    else { if (v4) REDUCE(T, true); else REDUCE(T, false); }
-#undef REDUCE
-    TF_CHECK_LAUNCH();
+  return launch_reduce<T>(st, p);
+}
+
+// One launch for a group of weight-gradient style products (both operands contraction-strided),
+// 256x256 tiles, direct-to-LDS kernel; then one reduce pass per problem.
+template <typename T>
+static int gemm_group_dispatch(hipStream_t st, const GemmGroup& g) {
+  constexpr int lds = 2 * (256 + 256) * 64 * 2;
+  auto kernel = gemm_dma_group_kernel<T, 256, 256, 64, 2, 4, 2, false, false>;
+  static bool once = (allow_big_lds(kernel, lds), true);
+  (void)once;
+  kernel<<<dim3((unsigned)g.first[g.count]), dim3(512), lds, st>>>(g);
+  TF_CHECK_LAUNCH();
+  for (int i = 0; i < g.count; ++i) {
+    const int rc = launch_reduce<T>(st, g.p[i]);
+    if (rc != TF_OK) return rc;
   }
   return TF_OK;
 }
@@ -924,4 +970,119 @@ extern "C" int tf_gemm_out_chunked(void* stream, int dtype, int out_dtype, int l
   hipStream_t st = (hipStream_t)stream;
   if (dtype == TF_F16) return gemm_dispatch<f16>(st, layout_a, layout_b, vec, pl, p);
   return gemm_dispatch<bf16>(st, layout_a, layout_b, vec, pl, p);
+}
+
+// ---- grouped products -------------------------------------------------------
+namespace {
+
+struct GroupPlan {
+  bool grouped;   // one launch for all problems (otherwise: one tf_gemm_out_chunked call each)
+  int splits;
+  int64_t need;   // workspace bytes
+};
+
+bool group_problem_ok(const tf_gemm_problem& q) {
+  return q.A && q.B && q.C && q.M > 0 && q.N > 0 && q.K > 0 && q.M <= 0x7fffff00 && q.N <= 0x7fffff00 &&
+         q.K <= 0x7fffff00;
+}
+
+// Fast-path preconditions of the direct-to-LDS kernel for a (K-minor, K-minor) problem.
+bool group_problem_fast(const tf_gemm_problem& q) {
+  const int64_t cn = (q.chunk_n <= 0 || q.chunk_n >= q.N) ? q.N : q.chunk_n;
+  return aligned16(q.A) && aligned16(q.B) && aligned16(q.C) && q.M % 8 == 0 && q.N % 8 == 0 && q.lda % 8 == 0 &&
+         q.ldb % 8 == 0 && q.ldc % 8 == 0 && q.K % 64 == 0 && q.lda >= q.M && q.ldb >= q.N && q.ldc >= cn &&
+         q.N % cn == 0 && cn % 8 == 0 && (cn == q.N || (q.chunk_stride % 8 == 0 && q.chunk_stride >= (q.M - 1) * q.ldc + cn));
+}
+
+GroupPlan plan_group(int la, int lb, int count, const tf_gemm_problem* pr) {
+  GroupPlan gp = {false, 1, 0};
+  bool fast = count >= 2 && count <= kMaxGroup && la == TF_OP_KMINOR && lb == TF_OP_KMINOR && g_force_cfg < 0 &&
+              g_force_splits <= 0;
+  int64_t tiles = 0, min_ksteps = INT64_MAX;
+  for (int i = 0; i < count && fast; ++i) {
+    fast = group_problem_ok(pr[i]) && group_problem_fast(pr[i]);
+    if (!fast) break;
+    tiles += ((pr[i].M + 255) / 256) * ((pr[i].N + 255) / 256);
+    const int64_t ks = pr[i].K / 64;
+    if (ks < min_ksteps) min_ksteps = ks;
+  }
+  if (fast && tiles < 0x7fffff) {
+    // same rule as for a single product: split only when the tiles alone leave most CUs idle,
+    // never beyond one round of workgroups, slices of at least 16 steps
+    int64_t splits = 1;
+    if (tiles <= 128) {
+      splits = 256 / tiles;
+      const int64_t max_by_k = min_ksteps / 16 > 0 ? min_ksteps / 16 : 1;
+      if (splits > max_by_k) splits = max_by_k;
+      if (splits > 16) splits = 16;
+    }
+    gp.grouped = true;
+    gp.splits = (int)splits;
+    if (splits > 1)
+      for (int i = 0; i < count; ++i) gp.need += splits * pr[i].M * pr[i].N * (int64_t)sizeof(float);
+    return gp;
+  }
+  for (int i = 0; i < count; ++i) {
+    if (!group_problem_ok(pr[i])) continue;
+    const int64_t n = tf_gemm_workspace_bytes(la, lb, pr[i].M, pr[i].N, pr[i].K);
+    if (n > gp.need) gp.need = n;
+  }
+  return gp;
+}
+
+}  // namespace
+
+extern "C" int64_t tf_gemm_group_workspace_bytes(int layout_a, int layout_b, int count, const tf_gemm_problem* problems) {
+  if (!problems || count < 1 || count > kMaxGroup) return 0;
+  return plan_group(layout_a, layout_b, count, problems).need;
+}
+
+extern "C" int tf_gemm_group(void* stream, int dtype, int out_dtype, int layout_a, int layout_b, int count,
+                             const tf_gemm_problem* problems, void* workspace, int64_t workspace_bytes) {
+  if (!problems || count < 1 || count > kMaxGroup) return TF_EINVAL;
+  if (dtype != TF_F16 && dtype != TF_BF16) return TF_EDTYPE;
+  if (out_dtype != dtype && out_dtype != TF_F32) return TF_EDTYPE;
+  const GroupPlan gp = plan_group(layout_a, layout_b, count, problems);
+  if (gp.need > 0 && (!workspace || workspace_bytes < gp.need)) return TF_EWORKSPACE;
+  if (!gp.grouped) {
+    for (int i = 0; i < count; ++i) {
+      const tf_gemm_problem& q = problems[i];
+      const int rc = tf_gemm_out_chunked(stream, dtype, out_dtype, layout_a, layout_b, q.M, q.N, q.K, q.A, q.lda, q.B,
+                                         q.ldb, q.C, q.ldc, q.chunk_n, q.chunk_stride, nullptr, 0, nullptr, 0,
+                                         workspace, workspace_bytes);
+      if (rc != TF_OK) return rc;
+    }
+    return TF_OK;
+  }
+  if (gp.need > 0 && !aligned16(workspace)) return TF_EALIGN;
+  GemmGroup g;
+  g.count = count;
+  g.first[0] = 0;
+  char* ws = (char*)workspace;
+  for (int i = 0; i < kMaxGroup; ++i) {
+    const tf_gemm_problem& q = problems[i < count ? i : 0];
+    GemmParams& p = g.p[i];
+    const int64_t cn = (q.chunk_n <= 0 || q.chunk_n >= q.N) ? q.N : q.chunk_n;
+    p.A = q.A; p.B = q.B; p.C = q.C; p.bias = nullptr; p.partial = (float*)ws;
+    p.M = (int)q.M; p.N = (int)q.N; p.K = (int)q.K;
+    p.lda = q.lda; p.ldb = q.ldb; p.ldc = q.ldc;
+    p.relu = 0;
+    p.tiles_m = (int)((q.M + 255) / 256); p.tiles_n = (int)((q.N + 255) / 256);
+    const int64_t ksteps = q.K / 64;
+    const int64_t steps_per = (ksteps + gp.splits - 1) / gp.splits;
+    p.k_per_split = (int)(steps_per * 64);
+    p.splits = (int)((ksteps + steps_per - 1) / steps_per);
+    p.flags = g_flags;
+    p.out_f32 = out_dtype == TF_F32 ? 1 : 0;
+    p.mask = nullptr; p.ldmask = 0;
+    p.chunk_n = (int)cn;
+    p.chunk_skip = (cn == q.N ? q.N : q.chunk_stride) - cn;
+    if (i < count) {
+      g.first[i + 1] = g.first[i] + p.tiles_m * p.tiles_n * p.splits;
+      if (p.splits > 1) ws += (int64_t)gp.splits * q.M * q.N * (int64_t)sizeof(float);
+    }
+  }
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == TF_F16) return gemm_group_dispatch<f16>(st, g);
+  return gemm_group_dispatch<bf16>(st, g);
 }

@@ -40,6 +40,16 @@ def _gemm(dtype, la, lb, m, n, k, a, lda, b, ldb, c, ldc, bias, relu, mask=None,
                                   ws.data_ptr() if ws is not None else None, ws_bytes))
 
 
+def _gemm_group(dtype, out_dtype, la, lb, problems, device):
+    """One tf_gemm_group call for a ctypes array of GemmProblem."""
+    lib = load()
+    n = len(problems)
+    ws_bytes = lib.tf_gemm_group_workspace_bytes(la, lb, n, problems)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=device) if ws_bytes else None
+    check(lib.tf_gemm_group(stream_ptr(), dtype_code(dtype), dtype_code(out_dtype), la, lb, n, problems,
+                            ws.data_ptr() if ws is not None else None, ws_bytes))
+
+
 def _check_linear(a, b, bias=None):
     # same preconditions as kernels/gemm.py:370-377, 584-591 of the reference
     if a.ndim != 3 or b.ndim != 2:
@@ -115,6 +125,41 @@ def mm_dw(x, grad, out_dtype=None, chunks=1):
     out = torch.empty((kin, nout), dtype=out_dtype or x.dtype, device=x.device)
     _gemm(x.dtype, KMINOR, KMINOR, kin, nout, t, x2, kin, g2, nout, out, nout, None, False)
     return out
+
+
+def mm_dw_group(pairs, out_dtype=None, chunks=None):
+    """``[mm_dw(x, g) for x, g in pairs]`` (up to four weight gradients that are available
+    at the same time) through ONE launch where the kernel's preconditions allow: products
+    whose outputs have few tiles then share the GPU instead of each splitting its contraction
+    into many slices.  ``chunks[i] > 1`` as in mm_dw."""
+    chunks = list(chunks) if chunks is not None else [1] * len(pairs)
+    if not 1 <= len(pairs) <= 4 or len(chunks) != len(pairs):
+        raise ValueError("mm_dw_group takes 1..4 (x, grad) pairs")
+    probs = (_lib.GemmProblem * len(pairs))()
+    outs, keep = [], []
+    dt = pairs[0][0].dtype
+    for i, ((x, grad), ch) in enumerate(zip(pairs, chunks)):
+        if x.shape[:-1] != grad.shape[:-1]:
+            raise ValueError("Leading dimensions of the two operands do not match")
+        if x.dtype != grad.dtype or x.dtype != dt:
+            raise TypeError("operands must share one 16-bit dtype")
+        require_cuda(x, grad)
+        x2, t, kin = _rows2d(x)
+        g2, _, nout = _rows2d(grad)
+        keep += [x2, g2]
+        if ch > 1:
+            if nout % ch or (nout // ch) % 8:
+                raise ValueError("column blocks must be equal and multiples of 8 wide")
+            each = nout // ch
+            out = torch.empty((ch, kin, each), dtype=out_dtype or dt, device=x.device)
+            ldc, cn, cs = each, each, kin * each
+        else:
+            out = torch.empty((kin, nout), dtype=out_dtype or dt, device=x.device)
+            ldc, cn, cs = nout, 0, 0
+        outs.append(out)
+        probs[i] = _lib.GemmProblem(kin, nout, t, x2.data_ptr(), kin, g2.data_ptr(), nout, out.data_ptr(), ldc, cn, cs)
+    _gemm_group(dt, outs[0].dtype, KMINOR, KMINOR, probs, outs[0].device)
+    return outs
 
 
 def cast_pack(weights, dtype):

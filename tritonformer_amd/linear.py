@@ -4,7 +4,11 @@ import torch
 from torch.autograd import Function
 
 from ._amp import amp_bwd, amp_fwd
-from .kernels import cast_pack, gemm, mask_grad, mm, mm_dw, unbroadcast_leading
+from .kernels import cast_pack, gemm, mask_grad, mm, mm_dw, mm_dw_group, unbroadcast_leading
+
+
+# True: weight gradients that are available together are computed by one grouped launch
+GROUP_DW = True
 
 
 def _grads(ctx, grad_output, inputs, weights):
@@ -117,10 +121,15 @@ class MLPReLU(Function):
         input, w1, w2, hidden = ctx.saved_tensors
         f32 = torch.float32
         grad_hidden = mm(grad_output, w2.T, mask_act=hidden)      # (dY W2^T) * (hidden > 0)
-        grad_w2 = mm_dw(hidden, grad_output, out_dtype=f32 if ctx.arg_dtypes[3] == f32 else None)
         grad_b2 = unbroadcast_leading(grad_output) if ctx.has_bias[1] else None
         grad_input = mm(grad_hidden, w1.T) if ctx.needs_input_grad[0] else None
-        grad_w1 = mm_dw(input, grad_hidden, out_dtype=f32 if ctx.arg_dtypes[1] == f32 else None)
+        if GROUP_DW and ctx.arg_dtypes[1] == ctx.arg_dtypes[3]:
+            # both weight gradients side by side in one launch
+            grad_w1, grad_w2 = mm_dw_group([(input, grad_hidden), (hidden, grad_output)],
+                                           out_dtype=f32 if ctx.arg_dtypes[1] == f32 else None)
+        else:
+            grad_w2 = mm_dw(hidden, grad_output, out_dtype=f32 if ctx.arg_dtypes[3] == f32 else None)
+            grad_w1 = mm_dw(input, grad_hidden, out_dtype=f32 if ctx.arg_dtypes[1] == f32 else None)
         grad_b1 = unbroadcast_leading(grad_hidden) if ctx.has_bias[0] else None
         return grad_input, grad_w1, grad_b1, grad_w2, grad_b2
 
