@@ -15,7 +15,7 @@ import torch
 
 import tritonformer_amd as T
 from oracle import ref_torch as R
-from tests.util import NUM_TEST, assert_close
+from tests.util import NUM_TEST, assert_close, rel_l2
 
 pytestmark = pytest.mark.gpu
 rng = np.random.RandomState(0)
@@ -150,3 +150,37 @@ def test_packed_qkv_equals_three_slices(use_bias, dev):
         assert torch.equal(a.grad[:, :, i].permute(0, 2, 1, 3), parts[i].grad)
     o_ref = R.causal_attention(*[p_.detach().cpu() for p_ in parts], bias.cpu() if use_bias else None)
     assert_close(out_s, o_ref, name="packed vs oracle")
+
+
+@pytest.mark.parametrize("use_bias", [False, True])
+def test_attention_block_equals_separate_functions(use_bias, dev):
+    """attention_block (projections + attention + output projection as one node) against
+    linear_no_bias_packed -> fast_causal_attention_qkvpacked -> linear_no_bias: the forward is
+    the same kernels in the same order (bitwise equal); gradients agree up to the fp32
+    summation order of the weight-gradient contraction (relative L2 < 1e-3 in fp16)."""
+    from tritonformer_amd.transformer import generate_alibi_mask
+
+    b, s, nh, hd = 2, 256, 4, 64
+    d = nh * hd
+    g = torch.Generator().manual_seed(21)
+    x = torch.randn(b, s, d, generator=g).half()
+    ws = [(torch.randn(d, d, generator=g) / d ** 0.5).half() for _ in range(4)]
+    dy = torch.randn(b, s, d, generator=g).half().to(dev)
+    bias = generate_alibi_mask(s, nh, device=dev)[0] if use_bias else None
+
+    def run(block):
+        xd = x.to(dev).requires_grad_(True)
+        wd = [w.to(dev).requires_grad_(True) for w in ws]
+        if block:
+            y = T.attention_block.apply(xd, *wd, nh, bias)
+        else:
+            qkv = T.linear_no_bias_packed.apply(xd, *wd[:3]).view(b, s, 3, nh, hd)
+            y = T.linear_no_bias.apply(T.fast_causal_attention_qkvpacked.apply(qkv, bias), wd[3])
+        y.backward(dy)
+        return y, xd.grad, [w.grad for w in wd]
+
+    y1, dx1, dw1 = run(True)
+    y0, dx0, dw0 = run(False)
+    assert torch.equal(y1, y0) and torch.equal(dx1, dx0)
+    for a, c in zip(dw1, dw0):
+        assert a.shape == (d, d) and a.is_contiguous() and rel_l2(a, c) < 1e-3

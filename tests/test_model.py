@@ -119,7 +119,7 @@ def test_unfused_reference_path_matches_fused(dev):
     model.load_state_dict(ref.state_dict())
     results = []
     for fuse in (True, False):
-        tr.FUSE_QKV = tr.FUSE_MLP = tr.FUSE_ADD_LN = fuse
+        tr.FUSE_QKV = tr.FUSE_MLP = tr.FUSE_ADD_LN = tr.FUSE_ATTN_BLOCK = fuse
         try:
             model.zero_grad(set_to_none=True)
             with torch.autocast("cuda", dtype=torch.float16):
@@ -127,7 +127,7 @@ def test_unfused_reference_path_matches_fused(dev):
             (loss * LOSS_SCALE).backward()
             results.append((loss.item(), {n: p.grad.clone() for n, p in model.named_parameters()}))
         finally:
-            tr.FUSE_QKV = tr.FUSE_MLP = tr.FUSE_ADD_LN = True
+            tr.FUSE_QKV = tr.FUSE_MLP = tr.FUSE_ADD_LN = tr.FUSE_ATTN_BLOCK = True
     assert abs(results[0][0] - results[1][0]) <= 1e-3 * abs(results[1][0])
     for n in results[0][1]:
         assert rel_l2(results[0][1][n], results[1][1][n]) < 2e-2, n

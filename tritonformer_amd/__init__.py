@@ -3,6 +3,7 @@ fattorib/tritonformer: the aliases below are the ones its ``__init__.py``
 exports, backed by hand-written HIP kernels behind a C ABI."""
 # The HIP library is loaded on the first kernel call (see _lib.load); if it has
 # not been built that call raises: there is no PyTorch or CPU fallback.
+from .attention import AttentionBlock as attention_block
 from .attention import BiasedCausalAttention as fast_causal_attention_with_bias
 from .attention import CausalAttention as fast_causal_attention
 from .attention import PackedCausalAttention as fast_causal_attention_qkvpacked

@@ -7,10 +7,13 @@ from torch.autograd import Function
 
 from ._amp import amp_bwd, amp_fwd
 from .kernels import (
+    cast_pack,
     flash_wrapper_bwd,
     flash_wrapper_bwd_attn_bias,
     flash_wrapper_fwd,
     flash_wrapper_fwd_attn_bias,
+    mm,
+    mm_dw_group,
 )
 
 
@@ -84,3 +87,46 @@ class PackedCausalAttention(Function):
         grad_output = grad_output.reshape(b, s, nh, hd).permute(0, 2, 1, 3)
         flash_wrapper_bwd(grad_output, out.permute(0, 2, 1, 3), q, k, v, lse, attn_bias, grads=grads)
         return dqkv, None
+
+
+class AttentionBlock(Function):
+    """The whole self-attention block of the reference model (transformer.py:153-190) as
+    ONE autograd node: ``apply(x, Wq, Wk, Wv, Wo, nh, attn_bias_or_None)`` =
+    ``attention(x Wq, x Wk, x Wv) Wo`` for bias-free projections (in, out) = (d, d).
+    Same GEMM and attention kernels as linear_no_bias_packed, fast_causal_attention_qkvpacked
+    and linear_no_bias one after the other; being one node, the weight gradients of the
+    packed q/k/v projection and of the output projection -- outputs with few tiles each --
+    are computed by one grouped launch."""
+
+    @staticmethod
+    @amp_fwd(keep=(1, 2, 3, 4))
+    def forward(ctx: Any, x, wq, wk, wv, wo, num_heads, attn_bias):
+        if x.ndim != 3 or wq.shape != (x.shape[-1], x.shape[-1]) or wo.shape != wq.shape:
+            raise ValueError("attention block takes x (B, S, d) and four (d, d) weights")
+        b, s, d = x.shape
+        hd = d // num_heads
+        w_qkv = cast_pack([wq, wk, wv], x.dtype)
+        w_o = cast_pack([wo], x.dtype)
+        qkv = mm(x, w_qkv).view(b, s, 3, num_heads, hd)
+        q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+        attn = torch.empty((b, s, num_heads, hd), dtype=x.dtype, device=x.device)
+        _, lse = flash_wrapper_fwd(q, k, v, attn_bias, out=attn.permute(0, 2, 1, 3))
+        attn = attn.view(b, s, d)
+        ctx.save_for_backward(x, w_qkv, w_o, qkv, attn, lse, attn_bias)
+        ctx.weight_dtype = wq.dtype
+        return mm(attn, w_o)
+
+    @staticmethod
+    @amp_bwd
+    def backward(ctx: Any, grad_output: torch.Tensor):
+        x, w_qkv, w_o, qkv, attn, lse, attn_bias = ctx.saved_tensors
+        b, s, _, nh, hd = qkv.shape
+        d_attn = mm(grad_output, w_o.T).view(b, s, nh, hd).permute(0, 2, 1, 3)
+        q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+        dqkv = torch.empty_like(qkv)
+        grads = tuple(dqkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+        flash_wrapper_bwd(d_attn, attn.view(b, s, nh, hd).permute(0, 2, 1, 3), q, k, v, lse, attn_bias, grads=grads)
+        dqkv = dqkv.view(b, s, 3 * nh * hd)
+        grad_x = mm(dqkv, w_qkv.T) if ctx.needs_input_grad[0] else None
+        d_wqkv, d_wo = mm_dw_group([(x, dqkv), (attn, grad_output)], out_dtype=ctx.weight_dtype, chunks=[3, 1])
+        return grad_x, d_wqkv[0], d_wqkv[1], d_wqkv[2], d_wo, None, None

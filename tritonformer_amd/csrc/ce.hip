@@ -57,18 +57,27 @@ __global__ __launch_bounds__(kCeThreads) void ce_fwd(int V, const T* __restrict_
   MaxSum acc = {-INFINITY, 0.f};
   if (VEC) {
     const int nchunk = V >> 3;
-    for (int c = threadIdx.x; c < nchunk; c += kCeThreads) {
-      float v[8];
-      Chunk<T>::load(xr + c * 8, v);
-      float cm = v[0];
+    constexpr int U = 4;  // 16-byte loads in flight per thread
+    for (int c0 = threadIdx.x; c0 < nchunk; c0 += U * kCeThreads) {
+      u32x4 raw[U];
 #pragma unroll
-      for (int e = 1; e < 8; ++e) cm = fmaxf(cm, v[e]);
-      cm *= kLog2e;
-      if (cm > acc.m) { acc.s *= exp2f(acc.m - cm); acc.m = cm; }
-      float part = 0.f;
+      for (int u = 0; u < U; ++u)
+        if (c0 + u * kCeThreads < nchunk) raw[u] = ld16(xr + (c0 + u * kCeThreads) * 8);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) part += exp2f(v[e] * kLog2e - acc.m);
-      acc.s += part;
+      for (int u = 0; u < U; ++u) {
+        if (c0 + u * kCeThreads >= nchunk) break;
+        float v[8];
+        unpack8<T>(raw[u], v);
+        float cm = v[0];
+#pragma unroll
+        for (int e = 1; e < 8; ++e) cm = fmaxf(cm, v[e]);
+        cm *= kLog2e;
+        if (cm > acc.m) { acc.s *= exp2f(acc.m - cm); acc.m = cm; }
+        float part = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) part += exp2f(v[e] * kLog2e - acc.m);
+        acc.s += part;
+      }
     }
   } else {
     for (int c = threadIdx.x; c < V; c += kCeThreads) {

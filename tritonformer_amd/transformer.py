@@ -20,6 +20,7 @@ import torch.nn as nn
 
 from . import (
     add_layer_norm,
+    attention_block,
     fast_causal_attention,
     fast_causal_attention_qkvpacked,
     fast_causal_attention_with_bias,
@@ -76,6 +77,9 @@ FUSE_QKV = True
 # True: the MLP block is one autograd node (ReLU gradient mask fused into a GEMM write-out);
 # False: two Linear modules as in the reference (transformer.py:214-217).
 FUSE_MLP = True
+# True (with FUSE_QKV): projections, attention and output projection are one autograd node, whose
+# two weight-gradient products run as one grouped launch.
+FUSE_ATTN_BLOCK = True
 # True: every residual addition runs inside the LayerNorm kernel that consumes its result
 # (forward), and the residual-stream gradient is added inside that LayerNorm's backward
 # kernel: no separate elementwise addition kernels.  False: `residual + hidden_states`
@@ -126,6 +130,9 @@ class CausalAttention(nn.Module):
 
     def forward(self, hidden_states: torch.Tensor, attn_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
         batch_size, q_seq_len, hidden_dim = hidden_states.shape
+        if FUSE_QKV and FUSE_ATTN_BLOCK:
+            return attention_block.apply(hidden_states, self.q_proj.weight, self.k_proj.weight, self.v_proj.weight,
+                                         self.out_proj.weight, self.num_attention_heads, attn_bias)
         if FUSE_QKV:
             # one (d, 3d) GEMM instead of three (d, d): same parameters, laid side by side in
             # 16 bits by one conversion kernel; the weight gradient comes back as three tensors
