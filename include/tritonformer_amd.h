@@ -127,7 +127,8 @@ int64_t tf_gemm_group_workspace_bytes(int layout_a, int layout_b, int count,
  * later tf_gemm / tf_gemm_workspace_bytes calls of this process. */
 int tf_gemm_tune(int cfg, int splits);
 /* Diagnostic: bit 0 disables the XCD-aware workgroup remap; bit 3 skips the
- * result write-out (WRONG results: it exists to time the main loop alone). */
+ * result write-out (WRONG results: it exists to time the main loop alone); bit 6
+ * disables the cut of a nearly empty last round of tiles into a split-contraction tail. */
 int tf_gemm_debug_flags(int flags);
 
 /* Causal flash attention forward.  q, k, v: logical (B, nh, S, hd) sharing the

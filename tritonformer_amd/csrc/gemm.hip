@@ -893,6 +893,31 @@ extern "C" int tf_gemm_debug_flags(int flags) {
   return TF_OK;
 }
 
+// A product whose 256x256 tiles fill a whole number of rounds of workgroups plus a small
+// remainder is cut in two along N: the columns that make whole rounds, and a narrow tail
+// that runs as a split contraction on the otherwise idle CUs instead of a nearly empty last
+// round (LM-head weight gradient: 4 x 197 tiles = 3 rounds + 20 tiles).  Returns the number
+// of tail columns, 0 for no cut.
+static int64_t tail_columns(int64_t M, int64_t N, int64_t K, bool vec, bool allow_split) {
+  if (!allow_split || g_force_cfg >= 0 || g_force_splits > 0 || K < 32 * 64 || (g_flags & 64)) return 0;
+  const GemmPlan pl = make_plan(M, N, K, vec, allow_split);
+  if (pl.cfg != 2 || pl.splits != 1) return 0;
+  const int64_t tiles = (int64_t)pl.tiles_m * pl.tiles_n;
+  const int64_t rem = tiles % 256;
+  if (tiles <= 256 || rem == 0 || rem > 64) return 0;
+  int64_t a = pl.tiles_m, b = 256;
+  while (b) { const int64_t t = a % b; a = b; b = t; }
+  const int64_t unit = 256 / a;  // tile columns per whole number of rounds
+  const int64_t tn1 = (pl.tiles_n / unit) * unit;
+  if (tn1 <= 0 || tn1 >= pl.tiles_n) return 0;
+  return N - tn1 * 256;
+}
+
+static int64_t single_need(int64_t M, int64_t N, int64_t K, bool vec) {
+  const GemmPlan pl = make_plan(M, N, K, vec);
+  return pl.splits > 1 ? (int64_t)pl.splits * M * N * (int64_t)sizeof(float) : 0;
+}
+
 extern "C" int64_t tf_gemm_workspace_bytes(int layout_a, int layout_b, int64_t M, int64_t N, int64_t K) {
   (void)layout_a;
   (void)layout_b;
@@ -900,8 +925,13 @@ extern "C" int64_t tf_gemm_workspace_bytes(int layout_a, int layout_b, int64_t M
   // the caller's alignment is unknown here: cover both kernel families
   int64_t need = 0;
   for (int vec = 0; vec < 2; ++vec) {
-    const GemmPlan pl = make_plan(M, N, K, vec != 0);
-    const int64_t n = pl.splits > 1 ? (int64_t)pl.splits * M * N * (int64_t)sizeof(float) : 0;
+    int64_t n = single_need(M, N, K, vec != 0);
+    const int64_t tail = tail_columns(M, N, K, vec != 0, true);
+    if (tail > 0) {
+      const int64_t n1 = single_need(M, N - tail, K, vec != 0), n2 = single_need(M, tail, K, vec != 0);
+      if (n1 > n) n = n1;
+      if (n2 > n) n = n2;
+    }
     if (n > need) need = n;
   }
   return need;
@@ -948,6 +978,22 @@ extern "C" int tf_gemm_out_chunked(void* stream, int dtype, int out_dtype, int l
   const bool vec = aligned16(A) && aligned16(B) && aligned16(C) && (!bias || aligned16(bias)) && a_contig % 8 == 0 &&
                    b_contig % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 && N % 8 == 0 && ldc % 8 == 0 &&
                    (!mask_act || (aligned16(mask_act) && ld_mask % 8 == 0));
+  if (chunk_n == N) {
+    const int64_t tail = tail_columns(M, N, K, vec, mask_act == nullptr);
+    if (tail > 0) {  // whole rounds first, then the narrow remainder as a split contraction
+      const int64_t n1 = N - tail;
+      const int64_t osz = out_dtype == TF_F32 ? 4 : 2;
+      const char* b2 = (const char*)B + (layout_b == TF_OP_KMAJOR ? n1 * ldb : n1) * 2;
+      const void* bias2 = bias ? (const char*)bias + n1 * 2 : nullptr;
+      const void* mask2 = mask_act ? (const char*)mask_act + n1 * 2 : nullptr;
+      const int rc = tf_gemm_out_chunked(stream, dtype, out_dtype, layout_a, layout_b, M, n1, K, A, lda, B, ldb, C, ldc,
+                                         0, 0, bias, relu, mask_act, ld_mask, workspace, workspace_bytes);
+      if (rc != TF_OK) return rc;
+      return tf_gemm_out_chunked(stream, dtype, out_dtype, layout_a, layout_b, M, tail, K, A, lda, b2, ldb,
+                                 (char*)C + n1 * osz, ldc, 0, 0, bias2, relu, mask2, ld_mask, workspace,
+                                 workspace_bytes);
+    }
+  }
   const GemmPlan pl = make_plan(M, N, K, vec, mask_act == nullptr);
   const int64_t need = pl.splits > 1 ? (int64_t)pl.splits * M * N * (int64_t)sizeof(float) : 0;
   if (need > 0 && (!workspace || workspace_bytes < need)) return TF_EWORKSPACE;
