@@ -29,7 +29,7 @@ PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per GEMM launch at the headline workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # scaled against a streaming kernel of known size (profiles/gemm_hbm_traffic_410m_step.md)
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = {"gpt2-410m-ctx2048-bs4": 152.8e6}
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = {"gpt2-410m-ctx2048-bs4": 171.9e6}
 
 WORKLOADS = {
     # name: (layers, d, heads, head_dim, ffn, seq, batch, linear_bias, alibi)
@@ -223,7 +223,7 @@ def main():
         achieved = gflops / (total_ms * 1e-3) / 1e12
         out["roofline"] = {
             "bound": "mfma",
-            "kernel": "tfa::gemm_dma_kernel (all instantiations; fwd X.W, dX = dY.W^T, dW = X^T.dY)",
+            "kernel": "tfa::gemm_dma_kernel / gemm_dma_group_kernel (all instantiations; fwd X.W, dX = dY.W^T, dW = X^T.dY)",
             "achieved": round(achieved, 2),
             "peak": PEAK_FP16_TFLOPS,
             "unit": "TFLOP/s",
