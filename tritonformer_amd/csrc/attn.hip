@@ -568,37 +568,81 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_dq
 #pragma unroll
     for (int r = 0; r < 16; ++r) dq[d][r] = 0.f;
 
-  u32x4 rk[KT::PER_THREAD], rv[KT::PER_THREAD];
-  KT::fetch(rk, K, p.ss, 0);
-  KT::fetch(rv, V, p.ss, 0);
-  KT::commit(smem, rk);
-  KT::commit(smem + KT::BYTES, rv);
+  // K and V tiles go from global memory straight into LDS, chunk swizzle on the global side
+  constexpr int PT = KT::PER_THREAD;
+  const T* kp[PT];
+#pragma unroll
+  for (int j = 0; j < PT; ++j) {
+    const int id = threadIdx.x + j * 256;
+    const int row = id / KT::CPR, c = (id % KT::CPR) ^ KT::swz(row);
+    kp[j] = K + (int64_t)row * p.ss + c * 8;
+  }
+  const int64_t v_minus_k = V - K;
+  auto load_tile = [&](int stage_off) {
+#pragma unroll
+    for (int j = 0; j < PT; ++j) {
+      char* dst = smem + stage_off + (j * 256 + wave * 64) * 16;
+      __builtin_amdgcn_global_load_lds((gptr_void*)kp[j], (lds_void*)dst, 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_void*)(kp[j] + v_minus_k), (lds_void*)(dst + KT::BYTES), 16, 0, 0);
+      kp[j] += (int64_t)64 * p.ss;
+    }
+  };
+  // lane-dependent parts of the LDS operand addresses (row operands of K and V, hd operands of K)
+  uint32_t ra[KS], ha[DT][2];
+  const uint32_t lds0 = lds_address(smem);
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) ra[ks] = lds0 + KT::addr(lane & 31, ks * 2 + (lane >> 5));
+#pragma unroll
+  for (int d = 0; d < DT; ++d) {
+    const int i = lane & 15;
+    const int col = d * 32 + 16 * ((lane >> 4) & 1) + (i & 3) * 4;
+    const int r0 = 4 * (lane >> 5) + (i >> 2);
+    ha[d][0] = lds0 + KT::addr(r0, col >> 3) + (col & 7) * 2;
+    ha[d][1] = lds0 + KT::addr(r0 + 8, col >> 3) + (col & 7) * 2;
+  }
+
+  load_tile(0);
   __syncthreads();
 
-  for (int j = 0; j < nkv; ++j) {
-    const char* sk = smem + (j & 1) * STAGE;
-    const char* sv = sk + KT::BYTES;
-    const bool more = j + 1 < nkv;
-    if (more) {
-      KT::fetch(rk, K, p.ss, (j + 1) * 64);
-      KT::fetch(rv, V, p.ss, (j + 1) * 64);
-    }
+  auto step = [&](auto stage_tag, int j) {
+    constexpr int SOFF = decltype(stage_tag)::value * STAGE;
+    if (j + 1 < nkv) load_tile(STAGE - SOFF);
     const int kb = j * 64;
     if (active) {
-#pragma unroll
-      for (int jt = 0; jt < 2; ++jt) {
+      static_for<2>([&](auto jt_tag) {
+        constexpr int jt = decltype(jt_tag)::value;
         const int ks0 = kb + jt * 32;  // first key of this 32-key sub-tile
-        if (ks0 > q0w + 31) continue;
+        if (ks0 > q0w + 31) return;
         auto tile = [&](auto diag_tag) {
           constexpr bool DIAG = decltype(diag_tag)::value;
+          // every operand of the sub-tile is requested before its first MFMA
+          constexpr int ROFF = SOFF + jt * 32 * HD * 2;
+          u32x4 kr[KS], vr[KS];
+          static_for<KS>([&](auto it) {
+            constexpr int ks = decltype(it)::value;
+            lds_read128_at<ROFF>(kr[ks], ra[ks]);
+            lds_read128_at<ROFF + KT::BYTES>(vr[ks], ra[ks]);
+          });
           f32x16 s, dp;
 #pragma unroll
           for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = neg_delta; }  // dP - delta for free
-#pragma unroll
-          for (int ks = 0; ks < KS; ++ks) {
-            s = mfma32(KT::frag_rows(sk, jt * 32, ks, lane), qf[ks], s);
-            dp = mfma32(KT::frag_rows(sv, jt * 32, ks, lane), dof[ks], dp);
-          }
+          static_for<KS>([&](auto it) {
+            constexpr int ks = decltype(it)::value;
+            constexpr int later_k = 2 * (KS - 1 - ks) + 1, later_v = later_k - 1;
+            lds_wait<(later_k < 15 ? later_k : 15)>(kr[ks]);
+            s = mfma32(__builtin_bit_cast(v8, kr[ks]), qf[ks], s);
+            lds_wait<(later_v < 15 ? later_v : 15)>(vr[ks]);
+            dp = mfma32(__builtin_bit_cast(v8, vr[ks]), dof[ks], dp);
+          });
+          // the hd-major K operands of dQ += dS K are requested now and arrive during the VALU work
+          constexpr int NH = 2 * DT;
+          u32x2 hlo[NH], hhi[NH];
+          static_for<NH>([&](auto it) {
+            constexpr int idx = decltype(it)::value, t = idx / DT, d = idx % DT;
+            constexpr int off = SOFF + (jt * 32 + t * 16) * HD * 2;
+            lds_read64_tr_at<off>(hlo[idx], ha[d][0]);
+            lds_read64_tr_at<off>(hhi[idx], ha[d][1]);
+          });
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
             const int key0 = ks0 + g * 8 + 4 * (lane >> 5);
@@ -618,23 +662,24 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_dq
               dp[g * 4 + e] *= pr;
             }
           }
-#pragma unroll
-          for (int t = 0; t < 2; ++t) {
+          static_for<NH>([&](auto it) {
+            constexpr int idx = decltype(it)::value, t = idx / DT, d = idx % DT;
+            constexpr int later = 2 * (NH - 1 - idx);
             const v8 dsb = round8<T>(dp, t);
-#pragma unroll
-            for (int d = 0; d < DT; ++d) dq[d] = mfma32(KT::frag_hd(sk, jt * 32 + t * 16, d, lane), dsb, dq[d]);
-          }
+            lds_wait<(later < 15 ? later : 15)>(hhi[idx]);
+            const u32x4 v = {hlo[idx][0], hlo[idx][1], hhi[idx][0], hhi[idx][1]};
+            dq[d] = mfma32(__builtin_bit_cast(v8, v), dsb, dq[d]);
+          });
         };
         if (ks0 + 31 > q0w) tile(std::true_type{});
         else tile(std::false_type{});
-      }
+      });
     }
-    if (more) {
-      char* dst = smem + ((j + 1) & 1) * STAGE;
-      KT::commit(dst, rk);
-      KT::commit(dst + KT::BYTES, rv);
-    }
-    __syncthreads();
+    __syncthreads();  // this thread's tile loads have landed, then everyone's; all reads of this stage are done
+  };
+  for (int j = 0; j < nkv; j += 2) {
+    step(std::integral_constant<int, 0>{}, j);
+    if (j + 1 < nkv) step(std::integral_constant<int, 1>{}, j + 1);
   }
 
   if (active) {
