@@ -114,6 +114,35 @@ __device__ __forceinline__ float max_with_other_half(float x) {
   return fmaxf(__builtin_bit_cast(float, r0), __builtin_bit_cast(float, r1));
 }
 
+// Additive-bias tile of a 128-query block and a 64-key block, 16 KB, staged through LDS with
+// coalesced direct-to-LDS loads: row r (128 bytes) keeps its 16-byte chunk c in slot
+// c ^ ((r >> 1) & 7), which spreads the 8-byte per-lane reads (one row per lane) over the banks.
+struct BiasTile {
+  static constexpr int BYTES = 128 * 64 * 2;
+  template <typename T>
+  static __device__ __forceinline__ void init(const T* (&bp)[4], const T* bias_head, int64_t row_stride, int q0, int S) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int id = threadIdx.x + j * 256;
+      const int row = id >> 3, c = (id & 7) ^ ((row >> 1) & 7);
+      const int qrow = min(q0 + row, S - 1);  // rows past the sequence are never read back
+      bp[j] = bias_head + (int64_t)qrow * row_stride + c * 8;
+    }
+  }
+  // next 64 keys into the tile at `dst`; advances the pointers
+  template <typename T> static __device__ __forceinline__ void load(const T* (&bp)[4], char* dst, int wave) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      __builtin_amdgcn_global_load_lds((gptr_void*)bp[j], (lds_void*)(dst + (j * 256 + wave * 64) * 16), 16, 0, 0);
+      bp[j] += 64;
+    }
+  }
+  // LDS address (relative to the tile) of keys chunk*8 + 4*half .. +3 of query row r
+  static __device__ __forceinline__ uint32_t addr(int r, int chunk, int half) {
+    return (uint32_t)(r * 128 + ((chunk ^ ((r >> 1) & 7)) << 4) + half * 8);
+  }
+};
+
 // Register r of a 32x32 MFMA result covers row (r/4)*8 + 4*(lane/32) + r%4.
 __device__ __forceinline__ int reg_row(int r, int lane) { return (r >> 2) * 8 + 4 * (lane >> 5) + (r & 3); }
 
@@ -133,12 +162,12 @@ __device__ __forceinline__ int reg_row(int r, int lane) { return (r >> 2) * 8 + 
 constexpr float kRescaleThreshold = 8.0f;  // log2 domain
 
 template <typename T, int HD, bool HAS_BIAS>
-__global__ __launch_bounds__(256, HD > 64 ? 1 : 3) void attn_fwd_kernel(AttnParams p) {
+__global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_fwd_kernel(AttnParams p) {
   typedef SeqTile<T, 64, HD> KT;
   typedef typename Vec<T>::v8 v8;
   typedef typename Vec<T>::v4 v4;
   constexpr int KS = HD / 16, DT = HD / 32;
-  constexpr int STAGE = 2 * KT::BYTES;
+  constexpr int STAGE = 2 * KT::BYTES + (HAS_BIAS ? BiasTile::BYTES : 0);
   constexpr int PT = KT::PER_THREAD;  // 16-byte chunks per thread per 64-row tile
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
@@ -160,7 +189,6 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : 3) void attn_fwd_kernel(AttnPara
   const int myq = q0w + (lane & 31);
   const int kv_end = min(p.S, q0 + 128);
   const int nkv = kv_end / 64;
-  const T* bias_row = HAS_BIAS ? (const T*)p.bias + (int64_t)h * p.bias_sh + (int64_t)myq * p.bias_sr : nullptr;
 
   v8 qf[KS];
 #pragma unroll
@@ -193,7 +221,9 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : 3) void attn_fwd_kernel(AttnPara
     kp[j] = K + (int64_t)row * p.ss + c * 8;
   }
   const int64_t v_minus_k = V - K;
-  auto load_tile = [&](int stage_off) {  // next 64 keys / values into the stage at byte offset stage_off
+  const T* bp[4];
+  if (HAS_BIAS) BiasTile::init(bp, (const T*)p.bias + (int64_t)h * p.bias_sh, p.bias_sr, q0, p.S);
+  auto load_tile = [&](int stage_off) {  // next 64 keys / values (/ bias columns) into the stage at byte offset stage_off
 #pragma unroll
     for (int j = 0; j < PT; ++j) {
       char* dst = smem + stage_off + (j * 256 + wave * 64) * 16;
@@ -201,6 +231,7 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : 3) void attn_fwd_kernel(AttnPara
       __builtin_amdgcn_global_load_lds((gptr_void*)(kp[j] + v_minus_k), (lds_void*)(dst + KT::BYTES), 16, 0, 0);
       kp[j] += (int64_t)64 * p.ss;
     }
+    if (HAS_BIAS) BiasTile::load(bp, smem + stage_off + 2 * KT::BYTES, wave);
   };
   // lane-dependent parts of the LDS operand addresses; block, sub-tile and stage offsets are
   // compile-time constants that end up in the instructions' offset fields
@@ -237,6 +268,16 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : 3) void attn_fwd_kernel(AttnPara
           constexpr int jt = decltype(it)::value % 2, ks = decltype(it)::value / 2;  // the two halves alternate
           lds_read128_at<SOFF + jt * 32 * HD * 2>(kf[jt][ks], ka[ks]);
         });
+        // ... and so are this lane's bias values: keys jt*32 + g*8 + 4*(lane/32) .. +3 of its query row
+        constexpr int NB = HAS_BIAS ? 8 : 0;
+        u32x2 braw[HAS_BIAS ? 8 : 1];
+        if constexpr (HAS_BIAS) {
+          const int r = wave * 32 + (lane & 31);
+          static_for<8>([&](auto it) {
+            constexpr int c = decltype(it)::value;  // 16-byte chunk = jt*4 + g
+            lds_read64_at<0>(braw[c], lds0 + (SOFF + 2 * KT::BYTES) + BiasTile::addr(r, c, lane >> 5));
+          });
+        }
         f32x16 st[2];
 #pragma unroll
         for (int jt = 0; jt < 2; ++jt)
@@ -244,19 +285,20 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : 3) void attn_fwd_kernel(AttnPara
           for (int r = 0; r < 16; ++r) st[jt][r] = 0.f;
         static_for<2 * KS>([&](auto it) {
           constexpr int idx = decltype(it)::value, jt = idx % 2, ks = idx / 2;  // two independent accumulation chains
-          lds_wait<2 * KS - 1 - idx>(kf[jt][ks]);
+          constexpr int later = 2 * KS - 1 - idx + NB;
+          lds_wait<(later < 15 ? later : 15)>(kf[jt][ks]);
           st[jt] = mfma32(__builtin_bit_cast(v8, kf[jt][ks]), qf[ks], st[jt]);
         });
         // block maximum; without bias it is taken over the raw scores and scaled once
         float mx = -INFINITY;
-#pragma unroll
-        for (int jt = 0; jt < 2; ++jt) {
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
+        static_for<8>([&](auto it) {
+          constexpr int jt = decltype(it)::value / 4, g = decltype(it)::value % 4;
+          {
             const int key0 = kb + jt * 32 + g * 8 + 4 * (lane >> 5);
             float bv[4] = {0.f, 0.f, 0.f, 0.f};
-            if (HAS_BIAS && (jt == 0 || live1)) {
-              const v4 raw = *reinterpret_cast<const v4*>(bias_row + key0);
+            if constexpr (HAS_BIAS) {
+              lds_wait<7 - decltype(it)::value>(braw[jt * 4 + g]);
+              const v4 raw = __builtin_bit_cast(v4, braw[jt * 4 + g]);
 #pragma unroll
               for (int e = 0; e < 4; ++e) bv[e] = (float)raw[e] * kLog2e;
             }
@@ -269,7 +311,7 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : 3) void attn_fwd_kernel(AttnPara
               mx = fmaxf(mx, x);
             }
           }
-        }
+        });
         // the V operands are requested now and arrive while the exponentials are computed
         constexpr int NVF = 4 * DT;  // operands of the block: (32-key half, 16-key step, 32-wide hd slice)
         u32x2 vlo[NVF], vhi[NVF];
@@ -524,7 +566,7 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_dq
   typedef typename Vec<T>::v8 v8;
   typedef typename Vec<T>::v4 v4;
   constexpr int KS = HD / 16, DT = HD / 32;
-  constexpr int STAGE = 2 * KT::BYTES;
+  constexpr int STAGE = 2 * KT::BYTES + (HAS_BIAS ? BiasTile::BYTES : 0);
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -578,6 +620,8 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_dq
     kp[j] = K + (int64_t)row * p.ss + c * 8;
   }
   const int64_t v_minus_k = V - K;
+  const T* bp[4];
+  if (HAS_BIAS) BiasTile::init(bp, (const T*)p.bias + (int64_t)h * p.bias_sh, p.bias_sr, q0, p.S);
   auto load_tile = [&](int stage_off) {
 #pragma unroll
     for (int j = 0; j < PT; ++j) {
@@ -586,6 +630,7 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_dq
       __builtin_amdgcn_global_load_lds((gptr_void*)(kp[j] + v_minus_k), (lds_void*)(dst + KT::BYTES), 16, 0, 0);
       kp[j] += (int64_t)64 * p.ss;
     }
+    if (HAS_BIAS) BiasTile::load(bp, smem + stage_off + 2 * KT::BYTES, wave);
   };
   // lane-dependent parts of the LDS operand addresses (row operands of K and V, hd operands of K)
   uint32_t ra[KS], ha[DT][2];
@@ -623,12 +668,22 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_dq
             lds_read128_at<ROFF>(kr[ks], ra[ks]);
             lds_read128_at<ROFF + KT::BYTES>(vr[ks], ra[ks]);
           });
+          // ... and this lane's bias values: keys jt*32 + g*8 + 4*(lane/32) .. +3 of its query row
+          constexpr int NB = HAS_BIAS ? 4 : 0;
+          u32x2 braw[HAS_BIAS ? 4 : 1];
+          if constexpr (HAS_BIAS) {
+            const int r = wave * 32 + (lane & 31);
+            static_for<4>([&](auto it) {
+              constexpr int g = decltype(it)::value;
+              lds_read64_at<0>(braw[g], lds0 + (SOFF + 2 * KT::BYTES) + BiasTile::addr(r, jt * 4 + g, lane >> 5));
+            });
+          }
           f32x16 s, dp;
 #pragma unroll
           for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = neg_delta; }  // dP - delta for free
           static_for<KS>([&](auto it) {
             constexpr int ks = decltype(it)::value;
-            constexpr int later_k = 2 * (KS - 1 - ks) + 1, later_v = later_k - 1;
+            constexpr int later_k = 2 * (KS - 1 - ks) + 1 + NB, later_v = later_k - 1;
             lds_wait<(later_k < 15 ? later_k : 15)>(kr[ks]);
             s = mfma32(__builtin_bit_cast(v8, kr[ks]), qf[ks], s);
             lds_wait<(later_v < 15 ? later_v : 15)>(vr[ks]);
@@ -643,13 +698,15 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_dq
             lds_read64_tr_at<off>(hlo[idx], ha[d][0]);
             lds_read64_tr_at<off>(hhi[idx], ha[d][1]);
           });
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
+          // (the bias values were requested before the hd-major operands: NH more reads are in flight)
+          static_for<4>([&](auto gt) {
+            constexpr int g = decltype(gt)::value;
             const int key0 = ks0 + g * 8 + 4 * (lane >> 5);
             float bv[4] = {0.f, 0.f, 0.f, 0.f};
-            if (HAS_BIAS) {
-              const v4 raw = *reinterpret_cast<const v4*>((const T*)p.bias + (int64_t)h * p.bias_sh +
-                                                          (int64_t)myq * p.bias_sr + key0);
+            if constexpr (HAS_BIAS) {
+              constexpr int later = 3 - g + 2 * NH;
+              lds_wait<(later < 15 ? later : 15)>(braw[g]);
+              const v4 raw = __builtin_bit_cast(v4, braw[g]);
 #pragma unroll
               for (int e = 0; e < 4; ++e) bv[e] = (float)raw[e] * kLog2e;
             }
@@ -661,7 +718,7 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_dq
               if (DIAG && key0 + e > myq) pr = 0.f;
               dp[g * 4 + e] *= pr;
             }
-          }
+          });
           static_for<NH>([&](auto it) {
             constexpr int idx = decltype(it)::value, t = idx / DT, d = idx % DT;
             constexpr int later = 2 * (NH - 1 - idx);
@@ -707,7 +764,7 @@ static void allow_lds(K kernel, int bytes) {
 
 template <typename T, int HD, bool HB>
 static int fwd_launch(hipStream_t st, const AttnParams& p) {
-  constexpr int lds = 4 * SeqTile<T, 64, HD>::BYTES;
+  constexpr int lds = 2 * (2 * SeqTile<T, 64, HD>::BYTES + (HB ? BiasTile::BYTES : 0));
   auto kernel = attn_fwd_kernel<T, HD, HB>;
   static bool once = (allow_lds(kernel, lds), true);
   (void)once;
@@ -733,7 +790,7 @@ static int bwd_launch(hipStream_t st, const AttnParams& p) {
     TF_CHECK_LAUNCH();
   }
   {
-    constexpr int lds = 4 * SeqTile<T, 64, HD>::BYTES;
+    constexpr int lds = 2 * (2 * SeqTile<T, 64, HD>::BYTES + (HB ? BiasTile::BYTES : 0));
     auto kernel = attn_dq_kernel<T, HD, HB>;
     static bool once = (allow_lds(kernel, lds), true);
     (void)once;
@@ -766,7 +823,7 @@ static int attn_check(int dtype, int64_t B, int64_t nh, int64_t S, int64_t hd, i
   if (B * nh * ((S + 127) / 128) > 0x7fffffff || S > (1 << 24)) return TF_EINVAL;
   if (sb % 8 || sh % 8 || ss % 8 || ss < hd) return TF_EALIGN;
   if (osb % 8 || osh % 8 || oss % 8 || oss < hd) return TF_EALIGN;
-  if (bias && (bias_sh % 4 || bias_sr % 4 || bias_sr < S)) return TF_EALIGN;
+  if (bias && (bias_sh % 8 || bias_sr % 8 || bias_sr < S)) return TF_EALIGN;
   return TF_OK;
 }
 
@@ -782,7 +839,7 @@ extern "C" int tf_attn_fwd(void* stream, int dtype, int64_t B, int64_t nh, int64
   const int rc = attn_check(dtype, B, nh, S, hd, sb, sh, ss, osb, osh, oss, bias, bias_sh, bias_sr);
   if (rc != TF_OK) return rc;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o)) return TF_EALIGN;
-  if (bias && (reinterpret_cast<uintptr_t>(bias) & 7)) return TF_EALIGN;
+  if (bias && (reinterpret_cast<uintptr_t>(bias) & 15)) return TF_EALIGN;
   AttnParams p = {};
   p.q = q; p.k = k; p.v = v; p.out = o; p.lse = lse; p.bias = bias;
   p.sb = sb; p.sh = sh; p.ss = ss; p.osb = osb; p.osh = osh; p.oss = oss;
@@ -805,7 +862,7 @@ extern "C" int tf_attn_bwd(void* stream, int dtype, int64_t B, int64_t nh, int64
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o) || !aligned16(d_o) || !aligned16(dq) ||
       !aligned16(dk) || !aligned16(dv))
     return TF_EALIGN;
-  if (bias && (reinterpret_cast<uintptr_t>(bias) & 7)) return TF_EALIGN;
+  if (bias && (reinterpret_cast<uintptr_t>(bias) & 15)) return TF_EALIGN;
   AttnParams p = {};
   p.q = q; p.k = k; p.v = v; p.o = o; p.d_o = d_o; p.dq = dq; p.dk = dk; p.dv = dv;
   p.lse = const_cast<float*>(lse); p.delta = delta; p.bias = bias;

@@ -100,12 +100,19 @@ __device__ __forceinline__ uint32_t lds_address(const char* p) {
   return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
 }
 template <int OFF> __device__ __forceinline__ void lds_read128_at(u32x4& dst, uint32_t addr) {
-  static_assert(OFF >= 0 && OFF < 65536, "offset field is 16 bits");
-  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+  static_assert(OFF >= 0, "offset");
+  constexpr int IMM = OFF < 65536 ? OFF : OFF % 32768;  // the instruction's offset field is 16 bits
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr + (uint32_t)(OFF - IMM)), "n"(IMM));
 }
 template <int OFF> __device__ __forceinline__ void lds_read64_tr_at(u32x2& dst, uint32_t addr) {
-  static_assert(OFF >= 0 && OFF < 65536, "offset field is 16 bits");
-  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+  static_assert(OFF >= 0, "offset");
+  constexpr int IMM = OFF < 65536 ? OFF : OFF % 32768;  // the instruction's offset field is 16 bits
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(dst) : "v"(addr + (uint32_t)(OFF - IMM)), "n"(IMM));
+}
+template <int OFF> __device__ __forceinline__ void lds_read64_at(u32x2& dst, uint32_t addr) {
+  static_assert(OFF >= 0, "offset");
+  constexpr int IMM = OFF < 65536 ? OFF : OFF % 32768;  // the instruction's offset field is 16 bits
+  asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(dst) : "v"(addr + (uint32_t)(OFF - IMM)), "n"(IMM));
 }
 template <int N, typename R> __device__ __forceinline__ void lds_wait(R& reg) {
   static_assert(N >= 0 && N <= 15, "lgkmcnt is 4 bits");

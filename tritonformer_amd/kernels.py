@@ -243,8 +243,12 @@ def _check_attn(q, k, v, bias):
 def _bias_args(bias):
     if bias is None:
         return None, None, 0, 0
-    if bias.stride(-1) != 1 or bias.stride(0) % 4 or bias.stride(1) % 4 or bias.data_ptr() % 8:
-        bias = bias.contiguous()
+    if bias.stride(-1) != 1 or bias.stride(0) % 8 or bias.stride(1) % 8 or bias.data_ptr() % 16:
+        # rows of whole 16-byte chunks: copy into storage whose row pitch is padded to 8 elements
+        nh, rows, cols = bias.shape
+        padded = torch.empty((nh, rows, (cols + 7) // 8 * 8), dtype=bias.dtype, device=bias.device)
+        padded[..., :cols].copy_(bias)
+        bias = padded[..., :cols]
     return bias, bias.data_ptr(), bias.stride(0), bias.stride(1)
 
 
