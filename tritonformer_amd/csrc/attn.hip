@@ -351,6 +351,7 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_fw
             constexpr int d = decltype(dd)::value, idx = (jt * 2 + t) * DT + d;
             constexpr int later = 2 * (NVF - 1 - idx);  // LDS reads requested after this operand
             lds_wait<(later < 15 ? later : 15)>(vhi[idx]);
+            lds_tie(vlo[idx]);
             const u32x4 v = {vlo[idx][0], vlo[idx][1], vhi[idx][0], vhi[idx][1]};
             oacc[d] = mfma32(__builtin_bit_cast(v8, v), pb, oacc[d]);
           });
@@ -384,7 +385,7 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_fw
 }
 
 // ===========================================================================
-// Backward pre-pass: delta[b,h,q] = sum_d dO[q,d] * O[q,d].
+// Backward pre-pass: delta[b,h,q] = -sum_d dO[q,d] * O[q,d] (stored negated).
 // ===========================================================================
 template <typename T, int HD>
 __global__ __launch_bounds__(256) void attn_delta_kernel(AttnParams p) {
@@ -404,7 +405,7 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(AttnParams p) {
   for (int e = 0; e < 8; ++e) acc += a[e] * g[e];
 #pragma unroll
   for (int o = LPR / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
-  if (threadIdx.x % LPR == 0) p.delta[row] = acc;
+  if (threadIdx.x % LPR == 0) p.delta[row] = -acc;  // negated: both consumers start dP from -delta
 }
 
 // ===========================================================================
@@ -417,7 +418,11 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_dkdv_kernel(AttnPa
   typedef typename Vec<T>::v8 v8;
   typedef typename Vec<T>::v4 v4;
   constexpr int KS = HD / 16, DT = HD / 32;
-  constexpr int STAGE = 2 * QT::BYTES + 2 * 64 * 4;
+  constexpr int PT = QT::PER_THREAD;
+  // one stage: Q tile, dO tile, lse[64] and -delta[64] (fp32), bias tile [64 queries][128 keys]
+  constexpr int STAT = 2 * QT::BYTES, BIAS = STAT + 2 * 64 * 4;
+  constexpr int BIAS_BYTES = 64 * 128 * 2;
+  constexpr int STAGE = BIAS + (HAS_BIAS ? BIAS_BYTES : 0);
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -430,8 +435,6 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_dkdv_kernel(AttnPa
   const T* K = (const T*)p.k + base;
   const T* V = (const T*)p.v + base;
   const T* dO = (const T*)p.d_o + (int64_t)b * p.osb + (int64_t)h * p.osh;
-  const float* lse = p.lse + (int64_t)bh * p.S;
-  const float* delta = p.delta + (int64_t)bh * p.S;
 
   const int k0 = kblk * 128;
   const int kw0 = k0 + wave * 32;
@@ -456,84 +459,177 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_dkdv_kernel(AttnPa
     for (int r = 0; r < 16; ++r) { dk[d][r] = 0.f; dv[d][r] = 0.f; }
 
   const int nq = (p.S - k0) / 64;  // query blocks k0, k0+64, ...
-  u32x4 rq[QT::PER_THREAD], rdo[QT::PER_THREAD];
-  float rstat = 0.f;  // threads 0..63: -lse, 64..127: -delta of the block's 64 queries
 
-  auto fetch = [&](int qb) {
-    QT::fetch(rq, Q, p.ss, qb);
-    QT::fetch(rdo, dO, p.oss, qb);
-    if (threadIdx.x < 64) rstat = -lse[qb + threadIdx.x];
-    else if (threadIdx.x < 128) rstat = -delta[qb + threadIdx.x - 64];
+  // Everything a query block needs goes from global memory straight into LDS: the Q and dO
+  // tiles (chunk swizzle on the global side), the two statistics rows (one float per lane of
+  // waves 0 and 1) and, with a bias, its [64][128] tile in plain row-major order.
+  const T* qp[PT];
+  const T* dop[PT];
+#pragma unroll
+  for (int j = 0; j < PT; ++j) {
+    const int id = threadIdx.x + j * 256;
+    const int row = id / QT::CPR, c = (id % QT::CPR) ^ QT::swz(row);
+    qp[j] = Q + (int64_t)(k0 + row) * p.ss + c * 8;
+    dop[j] = dO + (int64_t)(k0 + row) * p.oss + c * 8;
+  }
+  const float* statp = (wave == 0 ? p.lse : p.delta) + (int64_t)bh * p.S + k0 + lane;  // waves 0, 1 only
+  const T* bp[4];
+  if (HAS_BIAS) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int id = threadIdx.x + j * 256;
+      const int row = id >> 4;
+      int col = k0 + (id & 15) * 8;
+      if (col >= p.S) col = k0;  // keys past the sequence belong to inactive waves: any in-bounds column will do
+      bp[j] = (const T*)p.bias + (int64_t)h * p.bias_sh + (int64_t)(k0 + row) * p.bias_sr + col;
+    }
+  }
+  auto load_block = [&](int stage_off) {  // next 64 queries into the stage at byte offset stage_off
+#pragma unroll
+    for (int j = 0; j < PT; ++j) {
+      char* dst = smem + stage_off + (j * 256 + wave * 64) * 16;
+      __builtin_amdgcn_global_load_lds((gptr_void*)qp[j], (lds_void*)dst, 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_void*)dop[j], (lds_void*)(dst + QT::BYTES), 16, 0, 0);
+      qp[j] += (int64_t)64 * p.ss;
+      dop[j] += (int64_t)64 * p.oss;
+    }
+    if (wave < 2) {
+      __builtin_amdgcn_global_load_lds((gptr_void*)statp, (lds_void*)(smem + stage_off + STAT + wave * 256), 4, 0, 0);
+      statp += 64;
+    }
+    if (HAS_BIAS) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        __builtin_amdgcn_global_load_lds((gptr_void*)bp[j], (lds_void*)(smem + stage_off + BIAS + (j * 256 + wave * 64) * 16),
+                                         16, 0, 0);
+        bp[j] += (int64_t)64 * p.bias_sr;
+      }
+    }
   };
-  auto commit = [&](char* st) {
-    QT::commit(st, rq);
-    QT::commit(st + QT::BYTES, rdo);
-    if (threadIdx.x < 128) reinterpret_cast<float*>(st + 2 * QT::BYTES)[threadIdx.x] = rstat;
-  };
+  // lane-dependent parts of the LDS addresses
+  const uint32_t lds0 = lds_address(smem);
+  uint32_t ra[KS], ha[DT][2];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) ra[ks] = lds0 + QT::addr(lane & 31, ks * 2 + (lane >> 5));
+#pragma unroll
+  for (int d = 0; d < DT; ++d) {
+    const int i = lane & 15;
+    const int col = d * 32 + 16 * ((lane >> 4) & 1) + (i & 3) * 4;
+    const int r0 = 4 * (lane >> 5) + (i >> 2);
+    ha[d][0] = lds0 + QT::addr(r0, col >> 3) + (col & 7) * 2;
+    ha[d][1] = lds0 + QT::addr(r0 + 8, col >> 3) + (col & 7) * 2;
+  }
+  const uint32_t sa = lds0 + STAT + 16 * (lane >> 5);  // statistics of queries g*8 + 4*(lane/32) .. +3
+  const uint32_t ba = lds0 + BIAS + (4 * (lane >> 5)) * 256 + (wave * 32 + (lane & 31)) * 2;
 
-  if (nq > 0) { fetch(k0); commit(smem); }
+  if (nq > 0) load_block(0);
   __syncthreads();
 
-  for (int it = 0; it < nq; ++it) {
-    const char* sq = smem + (it & 1) * STAGE;
-    const char* sdo = sq + QT::BYTES;
-    const float* sstat = reinterpret_cast<const float*>(sq + 2 * QT::BYTES);
-    const bool more = it + 1 < nq;
+  auto step = [&](auto stage_tag, int it) {
+    constexpr int SOFF = decltype(stage_tag)::value * STAGE;
+    if (it + 1 < nq) load_block(STAGE - SOFF);
     const int qb = k0 + it * 64;
-    if (more) fetch(qb + 64);
     if (active) {
-#pragma unroll
-      for (int qt = 0; qt < 2; ++qt) {
+      static_for<2>([&](auto qt_tag) {
+        constexpr int qt = decltype(qt_tag)::value;
         const int qs = qb + qt * 32;      // first query of this 32-row sub-tile
-        if (qs + 31 < kw0) continue;      // entirely above the diagonal for this wave
+        if (qs + 31 < kw0) return;        // entirely above the diagonal for this wave
         auto tile = [&](auto diag_tag) {
           constexpr bool DIAG = decltype(diag_tag)::value;
-          // sstat holds -lse and -delta: dp starts at -delta, so dP - delta costs nothing
+          constexpr int ROFF = SOFF + qt * 32 * HD * 2;
+          // requests, in the order they are consumed: -delta (dP starts there, so dP - delta costs
+          // nothing), lse, then the row-major Q and dO operands
+          u32x4 dl[4], ls[4], qr[KS], dor[KS];
+          static_for<4>([&](auto g) {
+            lds_read128_at<SOFF + 256 + qt * 128 + decltype(g)::value * 32>(dl[decltype(g)::value], sa);
+          });
+          static_for<4>([&](auto g) {
+            lds_read128_at<SOFF + qt * 128 + decltype(g)::value * 32>(ls[decltype(g)::value], sa);
+          });
+          static_for<KS>([&](auto it2) {
+            constexpr int ks = decltype(it2)::value;
+            lds_read128_at<ROFF>(qr[ks], ra[ks]);
+            lds_read128_at<ROFF + QT::BYTES>(dor[ks], ra[ks]);
+          });
+          lds_wait<(2 * KS < 15 ? 2 * KS : 15)>(ls[3]);  // statistics have landed; the operands may be in flight
+          static_for<4>([&](auto g) { lds_tie(dl[decltype(g)::value]); lds_tie(ls[decltype(g)::value]); });
           f32x16 s, dp;
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
-            const f32x4 d4 = *reinterpret_cast<const f32x4*>(sstat + 64 + qt * 32 + g * 8 + 4 * (lane >> 5));
+            const f32x4 d4 = __builtin_bit_cast(f32x4, dl[g]);
 #pragma unroll
             for (int e = 0; e < 4; ++e) { s[g * 4 + e] = 0.f; dp[g * 4 + e] = d4[e]; }
           }
-#pragma unroll
-          for (int ks = 0; ks < KS; ++ks) {
-            s = mfma32(QT::frag_rows(sq, qt * 32, ks, lane), kf[ks], s);
-            dp = mfma32(QT::frag_rows(sdo, qt * 32, ks, lane), vf[ks], dp);
+          static_for<KS>([&](auto it2) {
+            constexpr int ks = decltype(it2)::value;
+            constexpr int later_q = 2 * (KS - 1 - ks) + 1;
+            lds_wait<(later_q < 15 ? later_q : 15)>(qr[ks]);
+            s = mfma32(__builtin_bit_cast(v8, qr[ks]), kf[ks], s);
+            lds_wait<(later_q - 1 < 15 ? later_q - 1 : 15)>(dor[ks]);
+            dp = mfma32(__builtin_bit_cast(v8, dor[ks]), vf[ks], dp);
+          });
+          // bias values, then the hd-major operands of the two accumulating products; they arrive
+          // during the exponentials
+          uint32_t braw[HAS_BIAS ? 16 : 1];
+          if constexpr (HAS_BIAS) {
+            static_for<16>([&](auto r) {
+              constexpr int g = decltype(r)::value / 4, e = decltype(r)::value % 4;
+              lds_read_u16_at<SOFF + (qt * 32 + g * 8 + e) * 256>(braw[decltype(r)::value], ba);
+            });
           }
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
+          constexpr int NH = 2 * DT;  // (16-query slice, 32-wide hd slice)
+          u32x2 dlo[NH], dhi[NH], qlo[NH], qhi[NH];
+          static_for<NH>([&](auto it2) {
+            constexpr int idx = decltype(it2)::value, t = idx / DT, d = idx % DT;
+            constexpr int off = SOFF + (qt * 32 + t * 16) * HD * 2;
+            lds_read64_tr_at<off + QT::BYTES>(dlo[idx], ha[d][0]);
+            lds_read64_tr_at<off + QT::BYTES>(dhi[idx], ha[d][1]);
+            lds_read64_tr_at<off>(qlo[idx], ha[d][0]);
+            lds_read64_tr_at<off>(qhi[idx], ha[d][1]);
+          });
+          if constexpr (HAS_BIAS) {
+            lds_wait<(4 * NH < 15 ? 4 * NH : 15)>(braw[15]);  // bias values have landed; operands may be in flight
+            static_for<15>([&](auto r) { lds_tie(braw[decltype(r)::value]); });
+          }
+          static_for<4>([&](auto gt) {
+            constexpr int g = decltype(gt)::value;
             const int ql = qt * 32 + g * 8 + 4 * (lane >> 5);  // block-local first query of the group
-            const f32x4 l4 = *reinterpret_cast<const f32x4*>(sstat + ql);
+            const f32x4 l4 = __builtin_bit_cast(f32x4, ls[g]);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               const int qi = qb + ql + e;
-              float x = fmaf(s[g * 4 + e], p.scale_log2, l4[e]);  // s*scale*log2e - lse
-              if (HAS_BIAS)
-                x += (float)((const T*)p.bias)[(int64_t)h * p.bias_sh + (int64_t)qi * p.bias_sr + mykey] * kLog2e;
+              float x = fmaf(s[g * 4 + e], p.scale_log2, -l4[e]);  // s*scale*log2e - lse
+              if constexpr (HAS_BIAS) x += (float)__builtin_bit_cast(T, (uint16_t)braw[g * 4 + e]) * kLog2e;
               float pr = fast_exp2(x);
               if (DIAG && mykey > qi) pr = 0.f;
               s[g * 4 + e] = pr;
               dp[g * 4 + e] *= pr;
             }
-          }
-#pragma unroll
-          for (int t = 0; t < 2; ++t) {
+          });
+          static_for<NH>([&](auto it2) {
+            constexpr int idx = decltype(it2)::value, t = idx / DT, d = idx % DT;
+            constexpr int later_d = 4 * (NH - 1 - idx) + 2, later_q = later_d - 2;
             const v8 pa = round8<T>(s, t);
             const v8 dsa = round8<T>(dp, t);
-#pragma unroll
-            for (int d = 0; d < DT; ++d) {
-              dv[d] = mfma32(QT::frag_hd(sdo, qt * 32 + t * 16, d, lane), pa, dv[d]);
-              dk[d] = mfma32(QT::frag_hd(sq, qt * 32 + t * 16, d, lane), dsa, dk[d]);
-            }
-          }
+            lds_wait<(later_d < 15 ? later_d : 15)>(dhi[idx]);
+            lds_tie(dlo[idx]);
+            const u32x4 a = {dlo[idx][0], dlo[idx][1], dhi[idx][0], dhi[idx][1]};
+            dv[d] = mfma32(__builtin_bit_cast(v8, a), pa, dv[d]);
+            lds_wait<(later_q < 15 ? later_q : 15)>(qhi[idx]);
+            lds_tie(qlo[idx]);
+            const u32x4 c = {qlo[idx][0], qlo[idx][1], qhi[idx][0], qhi[idx][1]};
+            dk[d] = mfma32(__builtin_bit_cast(v8, c), dsa, dk[d]);
+          });
         };
         if (qs < kw0 + 31) tile(std::true_type{});
         else tile(std::false_type{});
-      }
+      });
     }
-    if (more) commit(smem + ((it + 1) & 1) * STAGE);
-    __syncthreads();
+    __syncthreads();  // this thread's block loads have landed, then everyone's; all reads of this stage are done
+  };
+  for (int it = 0; it < nq; it += 2) {
+    step(std::integral_constant<int, 0>{}, it);
+    if (it + 1 < nq) step(std::integral_constant<int, 1>{}, it + 1);
   }
 
   if (active) {
@@ -602,7 +698,7 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_dq
   }
   if (active) {
     neg_lse = -p.lse[(int64_t)bh * p.S + myq];
-    neg_delta = -p.delta[(int64_t)bh * p.S + myq];
+    neg_delta = p.delta[(int64_t)bh * p.S + myq];  // the pre-pass stores it negated
   }
   f32x16 dq[DT];
 #pragma unroll
@@ -724,6 +820,7 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_dq
             constexpr int later = 2 * (NH - 1 - idx);
             const v8 dsb = round8<T>(dp, t);
             lds_wait<(later < 15 ? later : 15)>(hhi[idx]);
+            lds_tie(hlo[idx]);
             const u32x4 v = {hlo[idx][0], hlo[idx][1], hhi[idx][0], hhi[idx][1]};
             dq[d] = mfma32(__builtin_bit_cast(v8, v), dsb, dq[d]);
           });
@@ -782,7 +879,7 @@ static int bwd_launch(hipStream_t st, const AttnParams& p) {
   TF_CHECK_LAUNCH();
   const unsigned grid = (unsigned)(((p.S + 127) / 128) * p.B * p.nh);
   {
-    constexpr int lds = 2 * (2 * SeqTile<T, 64, HD>::BYTES + 2 * 64 * 4);
+    constexpr int lds = 2 * (2 * SeqTile<T, 64, HD>::BYTES + 2 * 64 * 4 + (HB ? 64 * 128 * 2 : 0));
     auto kernel = attn_dkdv_kernel<T, HD, HB>;
     static bool once = (allow_lds(kernel, lds), true);
     (void)once;

@@ -114,10 +114,20 @@ template <int OFF> __device__ __forceinline__ void lds_read64_at(u32x2& dst, uin
   constexpr int IMM = OFF < 65536 ? OFF : OFF % 32768;  // the instruction's offset field is 16 bits
   asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(dst) : "v"(addr + (uint32_t)(OFF - IMM)), "n"(IMM));
 }
+template <int OFF> __device__ __forceinline__ void lds_read_u16_at(uint32_t& dst, uint32_t addr) {
+  static_assert(OFF >= 0, "offset");
+  constexpr int IMM = OFF < 65536 ? OFF : OFF % 32768;
+  asm volatile("ds_read_u16 %0, %1 offset:%2" : "=v"(dst) : "v"(addr + (uint32_t)(OFF - IMM)), "n"(IMM));
+}
 template <int N, typename R> __device__ __forceinline__ void lds_wait(R& reg) {
   static_assert(N >= 0 && N <= 15, "lgkmcnt is 4 bits");
   asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(reg) : "n"(N));
 }
+
+// Orders every later use of `reg` after the preceding lds_wait (volatile asm statements keep
+// their order): for registers that were requested before the one the wait names and so have
+// landed with it.  Emits no instruction.
+template <typename R> __device__ __forceinline__ void lds_tie(R& reg) { asm volatile("" : "+v"(reg)); }
 
 // s_waitcnt vmcnt(n) with the other counters unconstrained (gfx9 encoding).
 template <int N> __device__ __forceinline__ void wait_vmcnt() {
