@@ -138,7 +138,8 @@ int tf_gemm_debug_flags(int flags);
  * also serve q, k, v that are slices of one packed (B, S, 3, nh, hd) buffer.)
  * lse: (B, nh, S) fp32, contiguous, log2-domain log-sum-exp of the scaled
  * (and biased) scores.  bias: NULL, or (nh, Sb, Sb) with Sb >= S, element
- * strides {bias_sh, bias_sr}, unit stride along keys, added after scaling
+ * strides {bias_sh, bias_sr} that are multiples of 8, 16-byte aligned, unit stride
+ * along keys, added after scaling
  * (kernels/biased_attention.py:101-106); -inf entries are allowed.
  * Replaces flash_wrapper_fwd (kernels/attention.py:171-217) and
  * flash_wrapper_fwd_attn_bias (kernels/biased_attention.py:188-245).
@@ -150,8 +151,8 @@ int tf_attn_fwd(void* stream, int dtype, int64_t B, int64_t nh, int64_t S, int64
                 float scale);
 
 /* Backward of the above: dq, dk, dv have q's strides, o and d_o the output
- * strides.  delta: (B, nh, S) fp32 scratch (row sums of dO*O), written then read
- * by this call.
+ * strides.  delta: (B, nh, S) fp32 scratch (negated row sums of dO*O), written then
+ * read by this call.
  * Replaces flash_wrapper_bwd (kernels/attention.py:550-607) and
  * flash_wrapper_bwd_attn_bias (kernels/biased_attention.py:598-660).
  * No gradient is produced for the bias (tritonformer/attention.py:60). */
