@@ -58,41 +58,44 @@ struct SeqTile {
   }
   static __device__ __forceinline__ int addr(int row, int chunk) { return (row * CPR + (chunk ^ swz(row))) * 16; }
 
-  // rows [row0, row0+ROWS) of a (seq, hd) matrix with row stride ss; always in bounds.
-  static __device__ __forceinline__ void fetch(u32x4 (&regs)[PER_THREAD], const T* __restrict__ base, int64_t ss,
-                                               int row0) {
+  // Direct-to-LDS loads: thread t's j-th 16-byte load lands in LDS slot t + 256 j of the tile,
+  // so the chunk swizzle is applied to the global address.  ptr[j] = address of that chunk in
+  // the tile whose first row is row0 of a (seq, hd) matrix with row stride ss.
+  static __device__ __forceinline__ void stream_init(const T* (&ptr)[PER_THREAD], const T* base, int64_t ss, int row0) {
 #pragma unroll
     for (int j = 0; j < PER_THREAD; ++j) {
       const int id = threadIdx.x + j * 256;
-      if (ROWS * CPR % 256 == 0 || id < ROWS * CPR) {
-        const int row = id / CPR, c = id % CPR;
-        regs[j] = ld16(base + (int64_t)(row0 + row) * ss + c * 8);
-      }
+      const int row = id / CPR, c = (id % CPR) ^ swz(row);
+      ptr[j] = base + (int64_t)(row0 + row) * ss + c * 8;
     }
   }
-  static __device__ __forceinline__ void commit(char* lds, const u32x4 (&regs)[PER_THREAD]) {
+  // LDS destination of a wave's j-th load into the tile at `tile`
+  static __device__ __forceinline__ char* stream_slot(char* tile, int wave, int j) {
+    return tile + (j * 256 + wave * 64) * 16;
+  }
+  // Lane-dependent parts of the LDS operand addresses of the tile at LDS address `tile`; block,
+  // sub-tile and stage offsets are compile-time constants that go into the offset fields.
+  static __device__ __forceinline__ void operand_addrs(uint32_t (&rows)[HD / 16], uint32_t (&hd)[HD / 32][2],
+                                                       uint32_t tile, int lane) {
 #pragma unroll
-    for (int j = 0; j < PER_THREAD; ++j) {
-      const int id = threadIdx.x + j * 256;
-      if (ROWS * CPR % 256 == 0 || id < ROWS * CPR) lds_st16(lds, addr(id / CPR, id % CPR), regs[j]);
+    for (int ks = 0; ks < HD / 16; ++ks) rows[ks] = tile + addr(lane & 31, ks * 2 + (lane >> 5));
+#pragma unroll
+    for (int d = 0; d < HD / 32; ++d) {
+      const int i = lane & 15;
+      const int col = d * 32 + 16 * ((lane >> 4) & 1) + (i & 3) * 4;
+      const int r0 = 4 * (lane >> 5) + (i >> 2);
+      hd[d][0] = tile + addr(r0, col >> 3) + (col & 7) * 2;
+      hd[d][1] = tile + addr(r0 + 8, col >> 3) + (col & 7) * 2;
     }
   }
-  // Operand with the tile's rows as the MFMA row/col index: lane l gets
-  // (row rb + l%32, hd = ks*16 + (l/32)*8 + 0..7).
-  static __device__ __forceinline__ v8 frag_rows(const char* lds, int rb, int ks, int lane) {
-    return __builtin_bit_cast(v8, lds_ld16(lds, addr(rb + (lane & 31), ks * 2 + (lane >> 5))));
-  }
-  // Operand with hd as the MFMA row/col index and the tile's rows as the
-  // contraction: lane l gets (hd = dt*32 + l%32, rows rb16 + 8*(s/4) + 4*(l/32) + s%4).
-  static __device__ __forceinline__ v8 frag_hd(const char* lds, int rb16, int dt, int lane) {
-    const int i = lane & 15;
-    const int col = dt * 32 + 16 * ((lane >> 4) & 1) + (i & 3) * 4;
-    const int r0 = rb16 + 4 * (lane >> 5) + (i >> 2);
-    const u32x2 lo = lds_ld8_tr(lds, addr(r0, col >> 3) + (col & 7) * 2);
-    const u32x2 hi = lds_ld8_tr(lds, addr(r0 + 8, col >> 3) + (col & 7) * 2);
-    u32x4 v = {lo[0], lo[1], hi[0], hi[1]};
-    return __builtin_bit_cast(v8, v);
-  }
+
+  // Operands read from a tile (the kernels issue the reads themselves, see below):
+  //  * rows as the MFMA row/col index: lane l reads 16 bytes at addr(rb + l%32, ks*2 + l/32),
+  //    i.e. (row rb + l%32, hd = ks*16 + (l/32)*8 + 0..7);
+  //  * hd as the MFMA row/col index, rows as the contraction: two transposing 8-byte reads at
+  //    addr(r0, col/8) + (col%8)*2 and the same 8 rows further down, with
+  //    col = dt*32 + 16*((l/16)%2) + (l%4)*4 and r0 = rb16 + 4*(l/32) + (l%16)/4; lane l ends up
+  //    with (hd = dt*32 + l%32, rows rb16 + 8*(s/4) + 4*(l/32) + s%4), s = 0..7.
 };
 
 template <typename T> __device__ __forceinline__ typename Vec<T>::v8 round8(const f32x16& x, int t) {
@@ -143,8 +146,7 @@ struct BiasTile {
   }
 };
 
-// Register r of a 32x32 MFMA result covers row (r/4)*8 + 4*(lane/32) + r%4.
-__device__ __forceinline__ int reg_row(int r, int lane) { return (r >> 2) * 8 + 4 * (lane >> 5) + (r & 3); }
+// (Register r of a 32x32 MFMA result covers row (r/4)*8 + 4*(lane/32) + r%4.)
 
 // ===========================================================================
 // Forward.  Workgroup: 4 waves x 32 queries; key/value blocks of 64.
@@ -158,6 +160,9 @@ __device__ __forceinline__ int reg_row(int r, int lane) { return (r >> 2) * 8 + 
 // core (an all-ones operand against P) instead of 32 VALU adds per row.
 // Occupancy: three waves per SIMD (168 VGPRs) for hd <= 64 without bias -- measured
 // 13 % faster than two, the third wave fills VALU/MFMA gaps of the other two.
+// K/V (and bias) tiles are loaded one block ahead straight into LDS; within a block all
+// K operands are requested before the first MFMA and all V operands before the
+// exponentials, as volatile-asm LDS reads with explicit waits (see common.h).
 // ===========================================================================
 constexpr float kRescaleThreshold = 8.0f;  // log2 domain
 
@@ -210,43 +215,25 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_fw
     for (int r = 0; r < 16; ++r) oacc[d][r] = 0.f;
   float m_ref = -INFINITY;  // reference maximum (log2 domain) the accumulators are scaled to
 
-  // K and V tiles go from global memory straight into LDS (no register staging): thread
-  // t's j-th 16-byte load lands in LDS slot t + 256 j of the tile, so the chunk swizzle of
-  // the tile layout is applied to the global address instead.
+  // K and V (and bias) tiles go from global memory straight into LDS, no register staging
   const T* kp[PT];
-#pragma unroll
-  for (int j = 0; j < PT; ++j) {
-    const int id = threadIdx.x + j * 256;
-    const int row = id / KT::CPR, c = (id % KT::CPR) ^ KT::swz(row);
-    kp[j] = K + (int64_t)row * p.ss + c * 8;
-  }
+  KT::stream_init(kp, K, p.ss, 0);
   const int64_t v_minus_k = V - K;
   const T* bp[4];
   if (HAS_BIAS) BiasTile::init(bp, (const T*)p.bias + (int64_t)h * p.bias_sh, p.bias_sr, q0, p.S);
   auto load_tile = [&](int stage_off) {  // next 64 keys / values (/ bias columns) into the stage at byte offset stage_off
 #pragma unroll
     for (int j = 0; j < PT; ++j) {
-      char* dst = smem + stage_off + (j * 256 + wave * 64) * 16;
-      __builtin_amdgcn_global_load_lds((gptr_void*)kp[j], (lds_void*)dst, 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((gptr_void*)(kp[j] + v_minus_k), (lds_void*)(dst + KT::BYTES), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_void*)kp[j], (lds_void*)KT::stream_slot(smem + stage_off, wave, j), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_void*)(kp[j] + v_minus_k),
+                                       (lds_void*)KT::stream_slot(smem + stage_off + KT::BYTES, wave, j), 16, 0, 0);
       kp[j] += (int64_t)64 * p.ss;
     }
     if (HAS_BIAS) BiasTile::load(bp, smem + stage_off + 2 * KT::BYTES, wave);
   };
-  // lane-dependent parts of the LDS operand addresses; block, sub-tile and stage offsets are
-  // compile-time constants that end up in the instructions' offset fields
   uint32_t ka[KS], va[DT][2];
   const uint32_t lds0 = lds_address(smem);
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks) ka[ks] = lds0 + KT::addr(lane & 31, ks * 2 + (lane >> 5));
-#pragma unroll
-  for (int d = 0; d < DT; ++d) {
-    const int i = lane & 15;
-    const int col = d * 32 + 16 * ((lane >> 4) & 1) + (i & 3) * 4;
-    const int r0 = 4 * (lane >> 5) + (i >> 2);
-    va[d][0] = lds0 + KT::addr(r0, col >> 3) + (col & 7) * 2;
-    va[d][1] = lds0 + KT::addr(r0 + 8, col >> 3) + (col & 7) * 2;
-  }
+  KT::operand_addrs(ka, va, lds0, lane);
 
   load_tile(0);
   __syncthreads();
@@ -465,13 +452,8 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_dkdv_kernel(AttnPa
   // waves 0 and 1) and, with a bias, its [64][128] tile in plain row-major order.
   const T* qp[PT];
   const T* dop[PT];
-#pragma unroll
-  for (int j = 0; j < PT; ++j) {
-    const int id = threadIdx.x + j * 256;
-    const int row = id / QT::CPR, c = (id % QT::CPR) ^ QT::swz(row);
-    qp[j] = Q + (int64_t)(k0 + row) * p.ss + c * 8;
-    dop[j] = dO + (int64_t)(k0 + row) * p.oss + c * 8;
-  }
+  QT::stream_init(qp, Q, p.ss, k0);
+  QT::stream_init(dop, dO, p.oss, k0);
   const float* statp = (wave == 0 ? p.lse : p.delta) + (int64_t)bh * p.S + k0 + lane;  // waves 0, 1 only
   const T* bp[4];
   if (HAS_BIAS) {
@@ -487,9 +469,9 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_dkdv_kernel(AttnPa
   auto load_block = [&](int stage_off) {  // next 64 queries into the stage at byte offset stage_off
 #pragma unroll
     for (int j = 0; j < PT; ++j) {
-      char* dst = smem + stage_off + (j * 256 + wave * 64) * 16;
-      __builtin_amdgcn_global_load_lds((gptr_void*)qp[j], (lds_void*)dst, 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((gptr_void*)dop[j], (lds_void*)(dst + QT::BYTES), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_void*)qp[j], (lds_void*)QT::stream_slot(smem + stage_off, wave, j), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_void*)dop[j], (lds_void*)QT::stream_slot(smem + stage_off + QT::BYTES, wave, j),
+                                       16, 0, 0);
       qp[j] += (int64_t)64 * p.ss;
       dop[j] += (int64_t)64 * p.oss;
     }
@@ -509,16 +491,7 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_dkdv_kernel(AttnPa
   // lane-dependent parts of the LDS addresses
   const uint32_t lds0 = lds_address(smem);
   uint32_t ra[KS], ha[DT][2];
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks) ra[ks] = lds0 + QT::addr(lane & 31, ks * 2 + (lane >> 5));
-#pragma unroll
-  for (int d = 0; d < DT; ++d) {
-    const int i = lane & 15;
-    const int col = d * 32 + 16 * ((lane >> 4) & 1) + (i & 3) * 4;
-    const int r0 = 4 * (lane >> 5) + (i >> 2);
-    ha[d][0] = lds0 + QT::addr(r0, col >> 3) + (col & 7) * 2;
-    ha[d][1] = lds0 + QT::addr(r0 + 8, col >> 3) + (col & 7) * 2;
-  }
+  QT::operand_addrs(ra, ha, lds0, lane);
   const uint32_t sa = lds0 + STAT + 16 * (lane >> 5);  // statistics of queries g*8 + 4*(lane/32) .. +3
   const uint32_t ba = lds0 + BIAS + (4 * (lane >> 5)) * 256 + (wave * 32 + (lane & 31)) * 2;
 
@@ -706,41 +679,27 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_dq
 #pragma unroll
     for (int r = 0; r < 16; ++r) dq[d][r] = 0.f;
 
-  // K and V tiles go from global memory straight into LDS, chunk swizzle on the global side
+  // K and V (and bias) tiles go from global memory straight into LDS
   constexpr int PT = KT::PER_THREAD;
   const T* kp[PT];
-#pragma unroll
-  for (int j = 0; j < PT; ++j) {
-    const int id = threadIdx.x + j * 256;
-    const int row = id / KT::CPR, c = (id % KT::CPR) ^ KT::swz(row);
-    kp[j] = K + (int64_t)row * p.ss + c * 8;
-  }
+  KT::stream_init(kp, K, p.ss, 0);
   const int64_t v_minus_k = V - K;
   const T* bp[4];
   if (HAS_BIAS) BiasTile::init(bp, (const T*)p.bias + (int64_t)h * p.bias_sh, p.bias_sr, q0, p.S);
   auto load_tile = [&](int stage_off) {
 #pragma unroll
     for (int j = 0; j < PT; ++j) {
-      char* dst = smem + stage_off + (j * 256 + wave * 64) * 16;
-      __builtin_amdgcn_global_load_lds((gptr_void*)kp[j], (lds_void*)dst, 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((gptr_void*)(kp[j] + v_minus_k), (lds_void*)(dst + KT::BYTES), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_void*)kp[j], (lds_void*)KT::stream_slot(smem + stage_off, wave, j), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_void*)(kp[j] + v_minus_k),
+                                       (lds_void*)KT::stream_slot(smem + stage_off + KT::BYTES, wave, j), 16, 0, 0);
       kp[j] += (int64_t)64 * p.ss;
     }
     if (HAS_BIAS) BiasTile::load(bp, smem + stage_off + 2 * KT::BYTES, wave);
   };
-  // lane-dependent parts of the LDS operand addresses (row operands of K and V, hd operands of K)
+  // row operands of K and V, hd operands of K
   uint32_t ra[KS], ha[DT][2];
   const uint32_t lds0 = lds_address(smem);
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks) ra[ks] = lds0 + KT::addr(lane & 31, ks * 2 + (lane >> 5));
-#pragma unroll
-  for (int d = 0; d < DT; ++d) {
-    const int i = lane & 15;
-    const int col = d * 32 + 16 * ((lane >> 4) & 1) + (i & 3) * 4;
-    const int r0 = 4 * (lane >> 5) + (i >> 2);
-    ha[d][0] = lds0 + KT::addr(r0, col >> 3) + (col & 7) * 2;
-    ha[d][1] = lds0 + KT::addr(r0 + 8, col >> 3) + (col & 7) * 2;
-  }
+  KT::operand_addrs(ra, ha, lds0, lane);
 
   load_tile(0);
   __syncthreads();
