@@ -157,6 +157,36 @@ def cpu_baseline(name, seconds_cap=60.0):
     }
 
 
+def mfma_probe(dtype, device, iters=20000):
+    """TFLOP/s of 256 workgroups x 8 waves issuing nothing but the GEMM step's MFMAs, per kind of operand data."""
+    from tritonformer_amd import _lib
+
+    lib = _lib.load()
+    sink = torch.empty(256 * 512, dtype=torch.float32, device=device)
+    gen = torch.Generator(device="cpu").manual_seed(0)
+    kinds = {
+        "all ones": torch.ones(24576),
+        "uniform in [-1, 1]": torch.rand(24576, generator=gen) * 2 - 1,
+        "normal, std 0.02 (weights)": torch.randn(24576, generator=gen) * 0.02,
+        "normal, std 1": torch.randn(24576, generator=gen),
+    }
+    out = {"probe": "v_mfma_f32_32x32x16 stream of one 256x256x64 GEMM step per trip, 256 workgroups x 8 waves, "
+                    "no memory traffic", "dtype": str(dtype).replace("torch.", ""), "iters": iters, "tflops": {}}
+    flops = lib.tf_probe_mfma_rate_flops(iters)
+    for name, vals in kinds.items():
+        ops = vals.to(dtype).to(device)
+        stream = torch.cuda.current_stream().cuda_stream
+        _lib.check(lib.tf_probe_mfma_rate(stream, _lib.dtype_code(dtype), ops.data_ptr(), 100, sink.data_ptr()))
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        _lib.check(lib.tf_probe_mfma_rate(stream, _lib.dtype_code(dtype), ops.data_ptr(), iters, sink.data_ptr()))
+        e1.record()
+        torch.cuda.synchronize()
+        out["tflops"][name] = round(flops / (e0.elapsed_time(e1) * 1e-3) / 1e12, 1)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -169,6 +199,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB streaming kernel, dst = src + 1 (known traffic: 1 GiB read, "
                          "1 GiB written) so that rocprofv3 FETCH_SIZE / WRITE_SIZE readings can be scaled")
+    ap.add_argument("--mfma-probe", action="store_true",
+                    help="instead of the step: sustained rate of the GEMM kernel's MFMA stream alone (no memory "
+                         "traffic) for constant and for random operand values, one JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported "
@@ -178,6 +211,9 @@ def main():
 
     dtype = torch.float16 if args.dtype == "fp16" else torch.bfloat16
     device = torch.device("cuda:0")
+    if args.mfma_probe:
+        print(json.dumps(mfma_probe(dtype, device)))
+        return
     L, d, nh, hd, f, S, B, lin_bias, alibi = WORKLOADS[args.workload]
     model, tokens = make_model(args.workload, device, dtype)
 

@@ -131,6 +131,15 @@ int tf_gemm_tune(int cfg, int splits);
  * disables the cut of a nearly empty last round of tiles into a split-contraction tail. */
 int tf_gemm_debug_flags(int flags);
 
+/* Diagnostic, no counterpart in the reference: the MFMA instruction stream of the
+ * 256x256x64 GEMM step alone (one workgroup per CU, 8 waves, no memory traffic),
+ * `iters` steps per workgroup, operands taken once from `operands` (8*6*64*8 = 24576
+ * elements of `dtype`, device memory); `sink`: 256*512 floats.  Time the call and divide
+ * tf_probe_mfma_rate_flops(iters) by it: the sustained rate depends on the operand
+ * values (the clock drops under the switching activity of random data). */
+int tf_probe_mfma_rate(void* stream, int dtype, const void* operands, int iters, float* sink);
+int64_t tf_probe_mfma_rate_flops(int iters);
+
 /* Causal flash attention forward.  q, k, v: logical (B, nh, S, hd) sharing the
  * element strides {sb, sh, ss}; o: the same logical shape with its own strides
  * {osb, osh, oss}; unit stride along hd everywhere.  (The reference passes q's

@@ -27,6 +27,8 @@ SIGNATURES = {
     "tf_gemm_out_chunked": (_i, [_vp, _i, _i, _i, _i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _i64, _i64,
                                  _vp, _i, _vp, _i64, _vp, _i64]),
     "tf_cast_pack": (_i, [_vp, _i, _i, _i, _i64, _i64, _vp, _i64, _vp, _i64]),
+    "tf_probe_mfma_rate": (_i, [_vp, _i, _vp, _i, _vp]),
+    "tf_probe_mfma_rate_flops": (_i64, [_i]),
     "tf_gemm_group": (_i, [_vp, _i, _i, _i, _i, _i, _vp, _vp, _i64]),
     "tf_gemm_group_workspace_bytes": (_i64, [_i, _i, _i, _vp]),
     "tf_gemm_workspace_bytes": (_i64, [_i, _i, _i64, _i64, _i64]),
