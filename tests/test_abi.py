@@ -94,6 +94,14 @@ def test_gemm_rejects_bad_arguments():
     assert lib.tf_cast_pack(None, 2, 0, 3, 0, 8, ptrs, 8, FAKE, 24) == 0           # nothing to do
 
 
+def test_probe_rejects_bad_arguments():
+    lib = _lib.load()
+    assert lib.tf_probe_mfma_rate(None, 0, None, 10, FAKE) == -1
+    assert lib.tf_probe_mfma_rate(None, 0, FAKE, 0, FAKE) == -1
+    assert lib.tf_probe_mfma_rate(None, 2, FAKE, 10, FAKE) == -2
+    assert lib.tf_probe_mfma_rate_flops(10) == 10 * 256 * 2 * 256 * 256 * 64
+
+
 def test_attention_rejects_bad_shapes():
     lib = _lib.load()
 
