@@ -225,6 +225,29 @@ int tf_add_layernorm_bwd(void* stream, int dtype, int param_dtype, int64_t rows,
 int tf_cast_pack(void* stream, int src_dtype, int dst_dtype, int count, int64_t rows, int64_t cols,
                  const void* const* srcs, int64_t ld_src, void* dst, int64_t ld_dst);
 
+/* Token (+ position) embedding, the part of the model the reference leaves to
+ * nn.Embedding (transformer.py:259-272, 311-323): out[t, :] = tok[ids[t], :] +
+ * pos[t mod S, :] for t < T (T = B*S whole sequences; `pos` may be null), added in
+ * fp32 and rounded once to out_dtype.  param_dtype TF_F32 with any out_dtype, or a
+ * 16-bit param_dtype with the same out_dtype.  tok is (V, d), pos (P, d), P >= S.
+ * An id outside [0, V) gives a row of zeros. */
+int tf_embedding_fwd(void* stream, int param_dtype, int out_dtype, int64_t T, int64_t S, int64_t d,
+                     int64_t V, int64_t P, const int64_t* ids, const void* tok, int64_t ld_tok,
+                     const void* pos, int64_t ld_pos, void* out, int64_t ld_out);
+
+/* Its backward: d_tok (V, d; contiguous, ld_dtok == d) = scatter-add of the rows of
+ * g (T, d) by token id, every other row zero; d_pos (P, d; may be null) = sum over
+ * sequences of g[b*S + s, :] for s < S, zero below.  fp32 accumulation in increasing
+ * position order, no atomics: bitwise reproducible.  Outputs are of param_dtype;
+ * grad_dtype any with TF_F32 parameters, else equal to param_dtype.  Gradient rows
+ * whose id lies outside [0, V) are dropped.  `workspace`: device memory of
+ * tf_embedding_bwd_workspace_bytes(T), 16-byte aligned. */
+int64_t tf_embedding_bwd_workspace_bytes(int64_t T);
+int tf_embedding_bwd(void* stream, int grad_dtype, int param_dtype, int64_t T, int64_t S, int64_t d,
+                     int64_t V, int64_t P, const int64_t* ids, const void* g, int64_t ld_g,
+                     void* d_tok, int64_t ld_dtok, void* d_pos, int64_t ld_dpos,
+                     void* workspace, int64_t workspace_bytes);
+
 /* Row softmax / its backward dx = y * (dy - sum(y*dy)); dtype f16/bf16/f32.
  * Replaces softmax_fwd / softmax_bwd (kernels/softmax.py:37-54, 95-111); the
  * backward writes a new buffer instead of overwriting grad_out. */

@@ -18,6 +18,8 @@ Pinning status (which independent check fixes each function):
   causal_attention          ref_ops.c loops (fwd + explicit bwd); SDPA(is_causal); row 0 = v[0];
                             zero bias == no bias
   get_slopes / alibi mask   closed forms for n = 8, 16, 24
+  embedding / _bwd          element loops on a tiny case (tests/test_oracle.py); F.embedding and
+                            its autograd; one-hot matrix product
   RefTransformer            zero-initialised LM head -> loss = ln(vocab) exactly and zero grads
                             upstream; parameter-name list; committed config-1 fixture
 No function of this oracle is "parity unpinned".
@@ -114,6 +116,28 @@ def causal_attention(q, k, v, bias=None):
 
 
 # --------------------------------------------------------------------------- ALiBi
+def embedding(ids, tok_w, pos_w=None):
+    """tok_w[ids] + pos_w[arange(S)] for (B, S) ids: reference transformer.py:311-323."""
+    out = tok_w.float()[ids]
+    if pos_w is not None:
+        out = out + pos_w.float()[torch.arange(ids.shape[1])][None]
+    return out
+
+
+def embedding_bwd(ids, g, vocab: int, positions: Optional[int] = None):
+    """Gradients of ``embedding``: rows of g (B, S, d) added up by token id -> (vocab, d), and
+    by position -> (positions, d) (rows >= S stay zero)."""
+    b, s = ids.shape
+    g = g.float()
+    d_tok = torch.zeros((vocab, g.shape[-1]), dtype=torch.float32)
+    d_tok.index_add_(0, ids.reshape(-1), g.reshape(b * s, -1))
+    if positions is None:
+        return d_tok, None
+    d_pos = torch.zeros((positions, g.shape[-1]), dtype=torch.float32)
+    d_pos[:s] = g.sum(0)
+    return d_tok, d_pos
+
+
 def get_slopes(n: int) -> List[float]:
     """reference transformer.py:37-52."""
     def pow2(m):

@@ -102,6 +102,28 @@ def test_probe_rejects_bad_arguments():
     assert lib.tf_probe_mfma_rate_flops(10) == 10 * 256 * 2 * 256 * 256 * 64
 
 
+def test_embedding_rejects_bad_arguments():
+    lib = _lib.load()
+
+    def fwd(T=8, S=4, d=16, V=10, P=4, ids=FAKE, pos=FAKE, pd=2, od=0, ld=16):
+        return lib.tf_embedding_fwd(None, pd, od, T, S, d, V, P, ids, FAKE, ld, pos, ld, FAKE, ld)
+
+    assert fwd(ids=None) == -1
+    assert fwd(T=7) == -4            # not whole sequences
+    assert fwd(P=3) == -4            # position table shorter than the sequence
+    assert fwd(pd=0, od=1) == -2     # 16-bit tables give their own dtype only
+    assert fwd(ld=8) == -1           # leading dimension shorter than a row
+
+    def bwd(T=8, S=4, d=16, V=10, P=4, ws=FAKE, nbytes=1 << 20, gd=0, pd=2, ldt=16):
+        return lib.tf_embedding_bwd(None, gd, pd, T, S, d, V, P, FAKE, FAKE, 16, FAKE, ldt, FAKE, 16, ws, nbytes)
+
+    assert lib.tf_embedding_bwd_workspace_bytes(8) == 64 and lib.tf_embedding_bwd_workspace_bytes(0) == 0
+    assert bwd(ws=None) == -5 and bwd(nbytes=63) == -5
+    assert bwd(T=6) == -4
+    assert bwd(ldt=32) == -1         # token gradient must be contiguous
+    assert bwd(gd=0, pd=1) == -2
+
+
 def test_attention_rejects_bad_shapes():
     lib = _lib.load()
 

@@ -180,6 +180,37 @@ def test_alibi_closed_forms():
     assert torch.equal(m[:, 5, 2], (torch.tensor(-3.0, dtype=torch.float16) * slopes))
 
 
+def test_embedding_vs_loops_and_library():
+    """The oracle's embedding and its gradient against element loops, F.embedding's autograd
+    and the one-hot matrix product (ids with repeats, so the scatter-add is exercised)."""
+    torch.manual_seed(3)
+    b, s, d, v, p = 2, 5, 3, 4, 7
+    ids = torch.randint(0, v, (b, s))
+    tok, pos = torch.randn(v, d), torch.randn(p, d)
+    out = R.embedding(ids, tok, pos)
+    for i in range(b):
+        for j in range(s):
+            for c in range(d):
+                assert out[i, j, c].item() == (tok[ids[i, j], c] + pos[j, c]).item()
+    assert torch.equal(R.embedding(ids, tok), tok[ids])
+    g = torch.randn(b, s, d)
+    d_tok, d_pos = R.embedding_bwd(ids, g, v, p)
+    loop_tok, loop_pos = torch.zeros(v, d, dtype=torch.float64), torch.zeros(p, d, dtype=torch.float64)
+    for i in range(b):
+        for j in range(s):
+            loop_tok[ids[i, j]] += g[i, j].double()
+            loop_pos[j] += g[i, j].double()
+    assert torch.allclose(d_tok.double(), loop_tok, atol=1e-6) and torch.allclose(d_pos.double(), loop_pos, atol=1e-6)
+    assert torch.count_nonzero(d_pos[s:]) == 0
+    tok_a, pos_a = tok.clone().requires_grad_(True), pos.clone().requires_grad_(True)
+    lib = F.embedding(ids, tok_a) + F.embedding(torch.arange(s)[None].expand(b, -1), pos_a)
+    assert torch.equal(lib, out)
+    lib.backward(g)
+    assert torch.allclose(tok_a.grad, d_tok, atol=1e-6) and torch.allclose(pos_a.grad, d_pos, atol=1e-6)
+    onehot = F.one_hot(ids.reshape(-1), v).float()
+    assert torch.allclose(onehot.T @ g.reshape(b * s, d), d_tok, atol=1e-6)
+
+
 def test_model_known_answers():
     cfg = R.RefConfig(50304, 64, 32, 2, 32, 128, 2, True, False)
     torch.manual_seed(0)

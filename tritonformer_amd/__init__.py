@@ -9,6 +9,7 @@ from .attention import CausalAttention as fast_causal_attention
 from .attention import PackedCausalAttention as fast_causal_attention_qkvpacked
 from .crossentropy import CrossEntropyLoss as cross_entropy_loss
 from .crossentropy import ShiftedCrossEntropyLoss as shifted_cross_entropy_loss
+from .embedding import EmbeddingSum as embedding_sum
 from .layernorm import AddLayerNorm as add_layer_norm
 from .layernorm import LayerNorm as layer_norm
 from .linear import LinearBias as linear_bias

@@ -27,6 +27,9 @@ SIGNATURES = {
     "tf_gemm_out_chunked": (_i, [_vp, _i, _i, _i, _i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _i64, _i64,
                                  _vp, _i, _vp, _i64, _vp, _i64]),
     "tf_cast_pack": (_i, [_vp, _i, _i, _i, _i64, _i64, _vp, _i64, _vp, _i64]),
+    "tf_embedding_fwd": (_i, [_vp, _i, _i, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _i64, _vp, _i64]),
+    "tf_embedding_bwd_workspace_bytes": (_i64, [_i64]),
+    "tf_embedding_bwd": (_i, [_vp, _i, _i, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64]),
     "tf_probe_mfma_rate": (_i, [_vp, _i, _vp, _i, _vp]),
     "tf_probe_mfma_rate_flops": (_i64, [_i]),
     "tf_gemm_group": (_i, [_vp, _i, _i, _i, _i, _i, _vp, _vp, _i64]),

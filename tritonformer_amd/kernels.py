@@ -180,6 +180,49 @@ def cast_pack(weights, dtype):
     return out
 
 
+def embedding_fwd(ids, tok_w, pos_w, out_dtype):
+    """(B, S) int64 ids -> (B, S, d): ``tok_w[ids] + pos_w[arange(S)]`` (``pos_w`` may be None),
+    added in fp32 and rounded once to ``out_dtype`` (reference transformer.py:311-323)."""
+    require_cuda(ids, tok_w)
+    if ids.ndim != 2 or ids.dtype != torch.int64 or tok_w.ndim != 2:
+        raise ValueError("embedding takes (B, S) int64 ids and a (V, d) table")
+    if pos_w is not None and (pos_w.ndim != 2 or pos_w.shape[1] != tok_w.shape[1] or pos_w.dtype != tok_w.dtype):
+        raise ValueError("position table must be (P, d) of the token table's dtype")
+    ids = ids.contiguous()
+    tok_w = tok_w if tok_w.stride(-1) == 1 else tok_w.contiguous()
+    if pos_w is not None and pos_w.stride(-1) != 1:
+        pos_w = pos_w.contiguous()
+    b, s = ids.shape
+    v, d = tok_w.shape
+    out = torch.empty((b, s, d), dtype=out_dtype, device=tok_w.device)
+    check(load().tf_embedding_fwd(stream_ptr(), dtype_code(tok_w.dtype), dtype_code(out_dtype), b * s, s, d, v,
+                                  0 if pos_w is None else pos_w.shape[0], ids.data_ptr(), tok_w.data_ptr(),
+                                  tok_w.stride(0), None if pos_w is None else pos_w.data_ptr(),
+                                  0 if pos_w is None else pos_w.stride(0), out.data_ptr(), d))
+    return out
+
+
+def embedding_bwd(grad_out, ids, tok_shape, pos_shape, param_dtype):
+    """Gradients of embedding_fwd's tables: (V, d) scatter-add by token id and, when
+    ``pos_shape`` is given, (P, d) sum over sequences; fp32 accumulation in position order."""
+    require_cuda(grad_out, ids)
+    ids = ids.contiguous()
+    b, s = ids.shape
+    v, d = tok_shape
+    g = grad_out.reshape(b * s, d)
+    if g.stride(-1) != 1:
+        g = g.contiguous()
+    lib = load()
+    d_tok = torch.empty((v, d), dtype=param_dtype, device=g.device)
+    d_pos = None if pos_shape is None else torch.empty(tuple(pos_shape), dtype=param_dtype, device=g.device)
+    nbytes = lib.tf_embedding_bwd_workspace_bytes(b * s)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=g.device)
+    check(lib.tf_embedding_bwd(stream_ptr(), dtype_code(g.dtype), dtype_code(param_dtype), b * s, s, d, v,
+                               0 if d_pos is None else d_pos.shape[0], ids.data_ptr(), g.data_ptr(), g.stride(0),
+                               d_tok.data_ptr(), d, None if d_pos is None else d_pos.data_ptr(), d, ws.data_ptr(), nbytes))
+    return d_tok, d_pos
+
+
 def unbroadcast_leading(x):
     """Sum over every dimension but the last, fp32 accumulation -> (cols,)
     (reference kernels/reductions.py:97-122)."""

@@ -21,6 +21,7 @@ import torch.nn as nn
 from . import (
     add_layer_norm,
     attention_block,
+    embedding_sum,
     fast_causal_attention,
     fast_causal_attention_qkvpacked,
     fast_causal_attention_with_bias,
@@ -85,6 +86,10 @@ FUSE_ATTN_BLOCK = True
 # kernel: no separate elementwise addition kernels.  False: `residual + hidden_states`
 # as the reference writes it (transformer.py:245-250).
 FUSE_ADD_LN = True
+# True: token gather, position gather, their addition and the rounding to the compute type are
+# one kernel, and the table gradients a chain-ordered scatter-add; False: two nn.Embedding
+# calls and an addition as in the reference (transformer.py:311-323).
+FUSE_EMBED = True
 
 
 def _weights_init(model: nn.Module, num_layers: int) -> None:
@@ -227,17 +232,23 @@ class Transformer(nn.Module):
 
     def forward(self, input_ids: torch.Tensor, labels: Optional[torch.Tensor]):
         batch_size, seq_len = input_ids.shape
-        hidden_states = self.embed_tokens(input_ids)
-        if self.embed_positions is not None:
-            positions = torch.arange(seq_len, device=hidden_states.device)[None].expand(batch_size, -1)
-            hidden_states = hidden_states + self.embed_positions(positions)
         attn_bias = self.attn_bias
-        if torch.is_autocast_enabled("cuda"):
-            # keep the residual stream in the 16-bit compute type, as it is in the
-            # reference (whose embeddings are fp16 parameters, transformer.py:259-272)
-            hidden_states = hidden_states.to(torch.get_autocast_dtype("cuda"))
-            if attn_bias is not None:
-                attn_bias = attn_bias.to(torch.get_autocast_dtype("cuda"))
+        # under autocast the residual stream is kept in the 16-bit compute type, as it is in
+        # the reference (whose embeddings are fp16 parameters, transformer.py:259-272)
+        amp_dtype = torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled("cuda") else None
+        if FUSE_EMBED and input_ids.is_cuda:
+            # gathers, addition and the rounding to the compute type in one kernel
+            pos_w = None if self.embed_positions is None else self.embed_positions.weight
+            hidden_states = embedding_sum.apply(input_ids, self.embed_tokens.weight, pos_w, amp_dtype)
+        else:
+            hidden_states = self.embed_tokens(input_ids)
+            if self.embed_positions is not None:
+                positions = torch.arange(seq_len, device=hidden_states.device)[None].expand(batch_size, -1)
+                hidden_states = hidden_states + self.embed_positions(positions)
+            if amp_dtype is not None:
+                hidden_states = hidden_states.to(amp_dtype)
+        if amp_dtype is not None and attn_bias is not None:
+            attn_bias = attn_bias.to(amp_dtype)
         if FUSE_ADD_LN and len(self.layer_list) > 0:
             pending = None
             for layer in self.layer_list:
