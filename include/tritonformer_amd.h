@@ -172,6 +172,23 @@ int tf_attn_bwd(void* stream, int dtype, int64_t B, int64_t nh, int64_t S, int64
                 const float* lse, float* delta,
                 const void* bias, int64_t bias_sh, int64_t bias_sr, float scale);
 
+/* tf_attn_fwd / tf_attn_bwd with the ALiBi bias of the reference's model in closed form
+ * instead of the dense (nh, S, S) matrix that generate_alibi_mask builds
+ * (transformer.py:37-75, 296-302; 805 MB at 24 heads x 4096): `slopes` = nh fp16 values
+ * (device memory), bias(h, i, j) = fp16(fp16(j - i) * slopes[h]) for j <= i -- distance,
+ * slope and product rounded to fp16 exactly as in that matrix, and the result rounded to
+ * bf16 when dtype is TF_BF16 (the matrix cast to the compute type) -- so the results are
+ * bit-identical to the dense calls on that matrix.  Other arguments as above. */
+int tf_attn_alibi_fwd(void* stream, int dtype, int64_t B, int64_t nh, int64_t S, int64_t hd,
+                      const void* q, const void* k, const void* v, void* o,
+                      int64_t sb, int64_t sh, int64_t ss, int64_t osb, int64_t osh, int64_t oss,
+                      float* lse, const void* slopes, float scale);
+int tf_attn_alibi_bwd(void* stream, int dtype, int64_t B, int64_t nh, int64_t S, int64_t hd,
+                      const void* q, const void* k, const void* v, const void* o, const void* d_o,
+                      void* dq, void* dk, void* dv,
+                      int64_t sb, int64_t sh, int64_t ss, int64_t osb, int64_t osh, int64_t oss,
+                      const float* lse, float* delta, const void* slopes, float scale);
+
 /* ---- bandwidth-bound kernels -------------------------------------------- */
 
 /* y = gamma * (x - mean) * rstd + beta over the last dimension; biased

@@ -140,6 +140,13 @@ def test_attention_rejects_bad_shapes():
     assert fwd(128, 64, bias=FAKE, bsr=64) == -3   # bias rows shorter than S
     assert lib.tf_attn_bwd(None, 0, 1, 2, 128, 64, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, None, 16384, 64, 128,
                            16384, 64, 128, FAKE, FAKE, None, 0, 0, 0.125) == -1  # null dv
+    # closed-form ALiBi: same checks, plus the slopes pointer
+    alibi = lambda S, hd, slopes: lib.tf_attn_alibi_fwd(None, 0, 1, 2, S, hd, FAKE, FAKE, FAKE, FAKE, S * 2 * hd, hd,
+                                                        2 * hd, S * 2 * hd, hd, 2 * hd, FAKE, slopes, 0.125)
+    assert alibi(128, 64, None) == -1 and alibi(128, 64, 0x1001) == -1
+    assert alibi(100, 64, FAKE) == -4 and alibi(128, 48, FAKE) == -4
+    assert lib.tf_attn_alibi_bwd(None, 0, 1, 2, 128, 64, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, 16384, 64, 128,
+                                 16384, 64, 128, FAKE, FAKE, None, 0.125) == -1
 
 
 def test_row_kernels_reject_bad_arguments():

@@ -39,13 +39,15 @@ def make_qkv(dims, dtype, dev, seed=0, strided=True):
     return q, k, v, do
 
 
-def run_case(dims, dtype, dev, bias=None, strided=True, seed=0):
+def run_case(dims, dtype, dev, bias=None, strided=True, seed=0, kernel_bias=None):
+    """``bias``: what the oracle adds; ``kernel_bias``: what the kernels are given for it when that
+    differs (the ALiBi slopes instead of the dense matrix)."""
     q, k, v, do = make_qkv(dims, dtype, dev, seed, strided)
     qd, kd, vd = (t.to(dev).requires_grad_(True) for t in (q, k, v))  # .to keeps the strides
     if bias is None:
         o = T.fast_causal_attention.apply(qd, kd, vd)
     else:
-        o = T.fast_causal_attention_with_bias.apply(qd, kd, vd, bias.to(dev))
+        o = T.fast_causal_attention_with_bias.apply(qd, kd, vd, (bias if kernel_bias is None else kernel_bias).to(dev))
     assert o.stride() == qd.stride() and o.dtype == dtype
     o.backward(do.to(dev))
     qr, kr, vr = (t.float().requires_grad_(True) for t in (q, k, v))

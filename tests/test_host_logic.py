@@ -5,6 +5,8 @@ import inspect
 import pytest
 import torch
 
+import tritonformer_amd.transformer as TM
+
 import tritonformer_amd as T
 from oracle import ref_torch as R
 from tritonformer_amd import nn as tnn
@@ -49,8 +51,18 @@ def test_parameter_names_and_shapes_match_oracle_model(bias, alibi):
     assert ("embed_positions.weight" in a) == (not alibi)
     assert a["layer_list.0.mlp.dense_h_to_4h.weight"] == (64, 128)
     ours.load_state_dict(ref.state_dict())  # interchangeable, buffers included
+    ref.load_state_dict(ours.state_dict())
     if alibi:
-        assert torch.equal(ours.attn_bias, ref.attn_bias)
+        # no dense matrix is kept (the kernels work from the slopes); a state dict still carries it
+        assert ours.attn_bias is None and ours.alibi_slopes.dtype == torch.float16
+        assert torch.equal(ours.state_dict()["attn_bias"], ref.attn_bias)
+        TM.FUSE_ALIBI = False
+        try:
+            dense = Transformer(cfg, device="cpu", param_dtype=torch.float32)
+        finally:
+            TM.FUSE_ALIBI = True
+        dense.load_state_dict(ours.state_dict())
+        assert dense.alibi_slopes is None and torch.equal(dense.attn_bias, ref.attn_bias)
 
 
 def test_initialisation_follows_reference():

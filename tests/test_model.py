@@ -17,6 +17,7 @@ import torch
 from oracle import ref_torch as R
 from tests.golden.make_config1_fixture import build_config1
 from tests.util import rel_l2
+import tritonformer_amd.transformer as TM
 from tritonformer_amd.transformer import Transformer, TransformerConfig
 
 pytestmark = pytest.mark.gpu
@@ -89,8 +90,27 @@ def test_alibi_model(dev):
     ids = torch.randint(0, 50304, (2, 128))      # seq 128 < max_position_embeddings 192
     model = Transformer(to_cfg(cfg), device=dev, param_dtype=torch.float32)
     model.load_state_dict(ref.state_dict())
-    assert model.embed_positions is None and model.attn_bias.shape == (4, 192, 192)
+    assert model.embed_positions is None and model.attn_bias is None and model.alibi_slopes.shape == (4,)
     compare(ref, model, ids, dev)
+    # the same with the dense (nh, S', S') matrix of the reference, larger than the sequence
+    TM.FUSE_ALIBI = False
+    try:
+        dense = Transformer(to_cfg(cfg), device=dev, param_dtype=torch.float32)
+    finally:
+        TM.FUSE_ALIBI = True
+    dense.load_state_dict(ref.state_dict())
+    assert dense.attn_bias.shape == (4, 192, 192)
+    ref.zero_grad(set_to_none=True)
+    compare(ref, dense, ids, dev)
+    # ... and the two agree bit for bit
+    results = []
+    for m in (model, dense):
+        m.zero_grad(set_to_none=True)
+        with torch.autocast("cuda", dtype=torch.float16):
+            _, loss = m(ids.to(dev), ids.to(dev))
+        loss.backward()
+        results.append((loss.item(), m.layer_list[0].attention.q_proj.weight.grad.clone()))
+    assert results[0][0] == results[1][0] and torch.equal(results[0][1], results[1][1])
 
 
 def test_step_is_deterministic(dev):

@@ -41,6 +41,10 @@ SIGNATURES = {
                          _vp, _vp, _i64, _i64, _f]),
     "tf_attn_bwd": (_i, [_vp, _i, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64,
                          _i64, _i64, _i64, _vp, _vp, _vp, _i64, _i64, _f]),
+    "tf_attn_alibi_fwd": (_i, [_vp, _i, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64,
+                               _vp, _vp, _f]),
+    "tf_attn_alibi_bwd": (_i, [_vp, _i, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64,
+                               _i64, _i64, _i64, _i64, _vp, _vp, _vp, _f]),
     "tf_layernorm_fwd": (_i, [_vp, _i, _i, _i64, _i64, _vp, _i64, _vp, _vp, _f, _vp, _i64, _vp, _vp]),
     "tf_layernorm_bwd": (_i, [_vp, _i, _i, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp,
                               _i64]),

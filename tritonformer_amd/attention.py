@@ -17,6 +17,15 @@ from .kernels import (
 )
 
 
+def _bias_for(attn_bias, dtype):
+    """A dense bias in the compute dtype (what autocast's cast of the argument would give);
+    ALiBi slopes -- a (nh,) vector -- stay float16, the precision the reference builds its
+    bias matrix from."""
+    if attn_bias is None or attn_bias.ndim == 1 or attn_bias.dtype == dtype:
+        return attn_bias
+    return attn_bias.to(dtype)
+
+
 class CausalAttention(Function):
     """softmax(causal(Q K^T / sqrt(hd))) V (reference attention.py:13-34)."""
 
@@ -37,7 +46,9 @@ class CausalAttention(Function):
 class BiasedCausalAttention(Function):
     """As CausalAttention with ``+ attn_bias[h, i, j]`` added to the scaled
     scores; no gradient for the bias (reference attention.py:37-60, which has no
-    autocast hook on this class)."""
+    autocast hook on this class).  Extension: ``attn_bias`` may be the (nh,) float16
+    vector of ALiBi slopes instead of the dense (nh, S, S) matrix built from them
+    (reference transformer.py:55-75); the results are the same bit for bit."""
 
     @staticmethod
     def forward(ctx: Any, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
@@ -63,10 +74,11 @@ class PackedCausalAttention(Function):
     separate projections, transformer.py:158-175)."""
 
     @staticmethod
-    @amp_fwd
+    @amp_fwd(keep=(1,))
     def forward(ctx: Any, qkv: torch.Tensor, attn_bias) -> torch.Tensor:
         if qkv.ndim != 5 or qkv.shape[2] != 3:
             raise ValueError("packed attention takes qkv of shape (B, S, 3, nh, hd)")
+        attn_bias = _bias_for(attn_bias, qkv.dtype)
         if not qkv.is_contiguous():
             qkv = qkv.contiguous()
         b, s, _, nh, hd = qkv.shape
@@ -99,10 +111,11 @@ class AttentionBlock(Function):
     are computed by one grouped launch."""
 
     @staticmethod
-    @amp_fwd(keep=(1, 2, 3, 4))
+    @amp_fwd(keep=(1, 2, 3, 4, 6))
     def forward(ctx: Any, x, wq, wk, wv, wo, num_heads, attn_bias):
         if x.ndim != 3 or wq.shape != (x.shape[-1], x.shape[-1]) or wo.shape != wq.shape:
             raise ValueError("attention block takes x (B, S, d) and four (d, d) weights")
+        attn_bias = _bias_for(attn_bias, x.dtype)
         b, s, d = x.shape
         hd = d // num_heads
         w_qkv = cast_pack([wq, wk, wv], x.dtype)

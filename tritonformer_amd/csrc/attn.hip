@@ -31,6 +31,7 @@ struct AttnParams {
   float* lse;    // written by fwd, read by bwd
   float* delta;  // written by the bwd pre-pass
   const void* bias;
+  const void* slopes;         // ALiBi in closed form: nh fp16 slopes instead of a dense bias
   int64_t sb, sh, ss;         // element strides of q, k, v and of dq, dk, dv
   int64_t osb, osh, oss;      // element strides of o and dO
   int64_t bias_sh, bias_sr;   // element strides of bias (head, query row)
@@ -117,6 +118,20 @@ __device__ __forceinline__ float max_with_other_half(float x) {
   return fmaxf(__builtin_bit_cast(float, r0), __builtin_bit_cast(float, r1));
 }
 
+// Bias modes of the kernels: none, a dense (nh, S', S') matrix, ALiBi in closed form.
+constexpr int kNoBias = 0, kDenseBias = 1, kAlibi = 2;
+
+// ALiBi bias of one (query, key) pair times log2(e), bit for bit what the dense path reads from
+// the matrix the reference builds (transformer.py:55-75): the distance key - query (<= 0) and the
+// slope are fp16 values, their product is rounded to fp16 once, a bf16 kernel sees that value
+// rounded to bf16 (the 16-bit matrix cast to the compute type).
+template <typename T> __device__ __forceinline__ float alibi_log2(float dist, _Float16 slope) {
+  const _Float16 b16 = (_Float16)dist * slope;
+  float b = (float)b16;
+  if (std::is_same<T, bf16>::value) b = (float)(T)b;
+  return b * kLog2e;
+}
+
 // Additive-bias tile of a 128-query block and a 64-key block, 16 KB, staged through LDS with
 // coalesced direct-to-LDS loads: row r (128 bytes) keeps its 16-byte chunk c in slot
 // c ^ ((r >> 1) & 7), which spreads the 8-byte per-lane reads (one row per lane) over the banks.
@@ -166,8 +181,9 @@ struct BiasTile {
 // ===========================================================================
 constexpr float kRescaleThreshold = 8.0f;  // log2 domain
 
-template <typename T, int HD, bool HAS_BIAS>
-__global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_fwd_kernel(AttnParams p) {
+template <typename T, int HD, int BMODE>
+__global__ __launch_bounds__(256, HD > 64 ? 1 : (BMODE == kDenseBias ? 2 : 3)) void attn_fwd_kernel(AttnParams p) {
+  constexpr bool HAS_BIAS = BMODE == kDenseBias, ALIBI = BMODE == kAlibi;
   typedef SeqTile<T, 64, HD> KT;
   typedef typename Vec<T>::v8 v8;
   typedef typename Vec<T>::v4 v4;
@@ -182,6 +198,7 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_fw
   const int qblk = nqb - 1 - (int)(blockIdx.x / nbh);  // heaviest query blocks first
   const int bh = blockIdx.x % nbh;
   const int b = bh / p.nh, h = bh % p.nh;
+  const _Float16 slope = ALIBI ? ((const _Float16*)p.slopes)[h] : (_Float16)0.f;
   const int64_t base = (int64_t)b * p.sb + (int64_t)h * p.sh;
   const T* Q = (const T*)p.q + base;
   const T* K = (const T*)p.k + base;
@@ -289,10 +306,15 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_fw
 #pragma unroll
               for (int e = 0; e < 4; ++e) bv[e] = (float)raw[e] * kLog2e;
             }
+            if constexpr (ALIBI) {
+              const float d0 = (float)(key0 - myq);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) bv[e] = alibi_log2<T>(d0 + (float)e, slope);
+            }
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               float x = st[jt][g * 4 + e];
-              if (HAS_BIAS) x = fmaf(x, p.scale_log2, bv[e]);
+              if (HAS_BIAS || ALIBI) x = fmaf(x, p.scale_log2, bv[e]);
               if (DIAG && (key0 + e > myq || (jt == 1 && !live1))) x = -INFINITY;
               st[jt][g * 4 + e] = x;
               mx = fmaxf(mx, x);
@@ -309,7 +331,7 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_fw
           lds_read64_tr_at<off>(vhi[idx], va[d][1]);
         });
         mx = max_with_other_half(mx);
-        if (!HAS_BIAS) mx *= p.scale_log2;  // scale > 0: max(s) * scale = max(s * scale)
+        if (!HAS_BIAS && !ALIBI) mx *= p.scale_log2;  // scale > 0: max(s) * scale = max(s * scale)
         // raise the reference maximum only when some row outgrew it by 2^8
         const bool grow = mx > m_ref + kRescaleThreshold;
         if (__any(grow)) {
@@ -328,7 +350,7 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_fw
         for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
           for (int r = 0; r < 16; ++r)
-            st[jt][r] = fast_exp2(HAS_BIAS ? st[jt][r] - m_use : fmaf(st[jt][r], p.scale_log2, -m_use));
+            st[jt][r] = fast_exp2((HAS_BIAS || ALIBI) ? st[jt][r] - m_use : fmaf(st[jt][r], p.scale_log2, -m_use));
         // every requested operand is consumed (a half above the diagonal contributes P = 0)
         static_for<4>([&](auto it) {
           constexpr int jt = decltype(it)::value / 2, t = decltype(it)::value % 2;
@@ -399,8 +421,9 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(AttnParams p) {
 // dK/dV pass.  Workgroup: 4 waves x 32 keys; query blocks of 64 from the
 // diagonal downwards.  Q and dO tiles (+ their lse / delta) go through LDS.
 // ===========================================================================
-template <typename T, int HD, bool HAS_BIAS>
+template <typename T, int HD, int BMODE>
 __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_dkdv_kernel(AttnParams p) {
+  constexpr bool HAS_BIAS = BMODE == kDenseBias, ALIBI = BMODE == kAlibi;
   typedef SeqTile<T, 64, HD> QT;
   typedef typename Vec<T>::v8 v8;
   typedef typename Vec<T>::v4 v4;
@@ -417,6 +440,7 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_dkdv_kernel(AttnPa
   const int kblk = (int)(blockIdx.x / nbh);  // lowest key blocks (longest loops) first
   const int bh = blockIdx.x % nbh;
   const int b = bh / p.nh, h = bh % p.nh;
+  const _Float16 slope = ALIBI ? ((const _Float16*)p.slopes)[h] : (_Float16)0.f;
   const int64_t base = (int64_t)b * p.sb + (int64_t)h * p.sh;
   const T* Q = (const T*)p.q + base;
   const T* K = (const T*)p.k + base;
@@ -573,6 +597,7 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_dkdv_kernel(AttnPa
               const int qi = qb + ql + e;
               float x = fmaf(s[g * 4 + e], p.scale_log2, -l4[e]);  // s*scale*log2e - lse
               if constexpr (HAS_BIAS) x += (float)__builtin_bit_cast(T, (uint16_t)braw[g * 4 + e]) * kLog2e;
+              if constexpr (ALIBI) x += alibi_log2<T>((float)(mykey - qi), slope);
               float pr = fast_exp2(x);
               if (DIAG && mykey > qi) pr = 0.f;
               s[g * 4 + e] = pr;
@@ -629,8 +654,9 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_dkdv_kernel(AttnPa
 // dQ pass.  Workgroup: 4 waves x 32 queries; key/value blocks of 64 up to the
 // diagonal, K and V tiles through LDS.
 // ===========================================================================
-template <typename T, int HD, bool HAS_BIAS>
-__global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_dq_kernel(AttnParams p) {
+template <typename T, int HD, int BMODE>
+__global__ __launch_bounds__(256, HD > 64 ? 1 : (BMODE != kNoBias ? 2 : 3)) void attn_dq_kernel(AttnParams p) {
+  constexpr bool HAS_BIAS = BMODE == kDenseBias, ALIBI = BMODE == kAlibi;
   typedef SeqTile<T, 64, HD> KT;
   typedef typename Vec<T>::v8 v8;
   typedef typename Vec<T>::v4 v4;
@@ -644,6 +670,7 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_dq
   const int qblk = nqb - 1 - (int)(blockIdx.x / nbh);
   const int bh = blockIdx.x % nbh;
   const int b = bh / p.nh, h = bh % p.nh;
+  const _Float16 slope = ALIBI ? ((const _Float16*)p.slopes)[h] : (_Float16)0.f;
   const int64_t base = (int64_t)b * p.sb + (int64_t)h * p.sh;
   const T* Q = (const T*)p.q + base;
   const T* K = (const T*)p.k + base;
@@ -765,10 +792,15 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (HAS_BIAS ? 2 : 3)) void attn_dq
 #pragma unroll
               for (int e = 0; e < 4; ++e) bv[e] = (float)raw[e] * kLog2e;
             }
+            if constexpr (ALIBI) {
+              const float d0 = (float)(key0 - myq);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) bv[e] = alibi_log2<T>(d0 + (float)e, slope);
+            }
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               float x = fmaf(s[g * 4 + e], p.scale_log2, neg_lse);
-              if (HAS_BIAS) x += bv[e];
+              if (HAS_BIAS || ALIBI) x += bv[e];
               float pr = fast_exp2(x);
               if (DIAG && key0 + e > myq) pr = 0.f;
               dp[g * 4 + e] *= pr;
@@ -818,10 +850,10 @@ static void allow_lds(K kernel, int bytes) {
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
 }
 
-template <typename T, int HD, bool HB>
+template <typename T, int HD, int MODE>
 static int fwd_launch(hipStream_t st, const AttnParams& p) {
-  constexpr int lds = 2 * (2 * SeqTile<T, 64, HD>::BYTES + (HB ? BiasTile::BYTES : 0));
-  auto kernel = attn_fwd_kernel<T, HD, HB>;
+  constexpr int lds = 2 * (2 * SeqTile<T, 64, HD>::BYTES + (MODE == kDenseBias ? BiasTile::BYTES : 0));
+  auto kernel = attn_fwd_kernel<T, HD, MODE>;
   static bool once = (allow_lds(kernel, lds), true);
   (void)once;
   const unsigned grid = (unsigned)(((p.S + 127) / 128) * p.B * p.nh);
@@ -830,7 +862,7 @@ static int fwd_launch(hipStream_t st, const AttnParams& p) {
   return TF_OK;
 }
 
-template <typename T, int HD, bool HB>
+template <typename T, int HD, int MODE>
 static int bwd_launch(hipStream_t st, const AttnParams& p) {
   const int64_t rows = (int64_t)p.B * p.nh * p.S;
   constexpr int rpb = 256 / (HD / 8);
@@ -838,16 +870,16 @@ static int bwd_launch(hipStream_t st, const AttnParams& p) {
   TF_CHECK_LAUNCH();
   const unsigned grid = (unsigned)(((p.S + 127) / 128) * p.B * p.nh);
   {
-    constexpr int lds = 2 * (2 * SeqTile<T, 64, HD>::BYTES + 2 * 64 * 4 + (HB ? 64 * 128 * 2 : 0));
-    auto kernel = attn_dkdv_kernel<T, HD, HB>;
+    constexpr int lds = 2 * (2 * SeqTile<T, 64, HD>::BYTES + 2 * 64 * 4 + (MODE == kDenseBias ? 64 * 128 * 2 : 0));
+    auto kernel = attn_dkdv_kernel<T, HD, MODE>;
     static bool once = (allow_lds(kernel, lds), true);
     (void)once;
     kernel<<<dim3(grid), dim3(256), lds, st>>>(p);
     TF_CHECK_LAUNCH();
   }
   {
-    constexpr int lds = 2 * (2 * SeqTile<T, 64, HD>::BYTES + (HB ? BiasTile::BYTES : 0));
-    auto kernel = attn_dq_kernel<T, HD, HB>;
+    constexpr int lds = 2 * (2 * SeqTile<T, 64, HD>::BYTES + (MODE == kDenseBias ? BiasTile::BYTES : 0));
+    auto kernel = attn_dq_kernel<T, HD, MODE>;
     static bool once = (allow_lds(kernel, lds), true);
     (void)once;
     kernel<<<dim3(grid), dim3(256), lds, st>>>(p);
@@ -856,18 +888,21 @@ static int bwd_launch(hipStream_t st, const AttnParams& p) {
   return TF_OK;
 }
 
-template <typename T, bool FWD>
-static int attn_dispatch(hipStream_t st, int hd, bool has_bias, const AttnParams& p) {
-#define GO(HD)                                                                          \
-  return FWD ? (has_bias ? fwd_launch<T, HD, true>(st, p) : fwd_launch<T, HD, false>(st, p)) \
-             : (has_bias ? bwd_launch<T, HD, true>(st, p) : bwd_launch<T, HD, false>(st, p))
+template <typename T, bool FWD, int MODE>
+static int attn_dispatch_hd(hipStream_t st, int hd, const AttnParams& p) {
   switch (hd) {
-    case 32: GO(32);
-    case 64: GO(64);
-    case 128: GO(128);
+    case 32: return FWD ? fwd_launch<T, 32, MODE>(st, p) : bwd_launch<T, 32, MODE>(st, p);
+    case 64: return FWD ? fwd_launch<T, 64, MODE>(st, p) : bwd_launch<T, 64, MODE>(st, p);
+    case 128: return FWD ? fwd_launch<T, 128, MODE>(st, p) : bwd_launch<T, 128, MODE>(st, p);
   }
-#undef GO
   return TF_ESHAPE;
+}
+
+template <typename T, bool FWD>
+static int attn_dispatch(hipStream_t st, int hd, const AttnParams& p) {
+  if (p.slopes) return attn_dispatch_hd<T, FWD, kAlibi>(st, hd, p);
+  if (p.bias) return attn_dispatch_hd<T, FWD, kDenseBias>(st, hd, p);
+  return attn_dispatch_hd<T, FWD, kNoBias>(st, hd, p);
 }
 
 static int attn_check(int dtype, int64_t B, int64_t nh, int64_t S, int64_t hd, int64_t sb, int64_t sh, int64_t ss,
@@ -887,31 +922,31 @@ static int attn_check(int dtype, int64_t B, int64_t nh, int64_t S, int64_t hd, i
 
 using namespace tfa;
 
-extern "C" int tf_attn_fwd(void* stream, int dtype, int64_t B, int64_t nh, int64_t S, int64_t hd, const void* q,
-                           const void* k, const void* v, void* o, int64_t sb, int64_t sh, int64_t ss, int64_t osb,
-                           int64_t osh, int64_t oss, float* lse, const void* bias, int64_t bias_sh, int64_t bias_sr,
-                           float scale) {
+static int attn_fwd_entry(void* stream, int dtype, int64_t B, int64_t nh, int64_t S, int64_t hd, const void* q,
+                          const void* k, const void* v, void* o, int64_t sb, int64_t sh, int64_t ss, int64_t osb,
+                          int64_t osh, int64_t oss, float* lse, const void* bias, int64_t bias_sh, int64_t bias_sr,
+                          const void* slopes, float scale) {
   if (!q || !k || !v || !o || !lse) return TF_EINVAL;
   const int rc = attn_check(dtype, B, nh, S, hd, sb, sh, ss, osb, osh, oss, bias, bias_sh, bias_sr);
   if (rc != TF_OK) return rc;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o)) return TF_EALIGN;
   if (bias && (reinterpret_cast<uintptr_t>(bias) & 15)) return TF_EALIGN;
   AttnParams p = {};
-  p.q = q; p.k = k; p.v = v; p.out = o; p.lse = lse; p.bias = bias;
+  p.q = q; p.k = k; p.v = v; p.out = o; p.lse = lse; p.bias = bias; p.slopes = slopes;
   p.sb = sb; p.sh = sh; p.ss = ss; p.osb = osb; p.osh = osh; p.oss = oss;
   p.bias_sh = bias_sh; p.bias_sr = bias_sr;
   p.B = (int)B; p.nh = (int)nh; p.S = (int)S;
   p.scale = scale; p.scale_log2 = scale * kLog2e;
   hipStream_t st = (hipStream_t)stream;
-  if (dtype == TF_F16) return attn_dispatch<f16, true>(st, (int)hd, bias != nullptr, p);
-  return attn_dispatch<bf16, true>(st, (int)hd, bias != nullptr, p);
+  if (dtype == TF_F16) return attn_dispatch<f16, true>(st, (int)hd, p);
+  return attn_dispatch<bf16, true>(st, (int)hd, p);
 }
 
-extern "C" int tf_attn_bwd(void* stream, int dtype, int64_t B, int64_t nh, int64_t S, int64_t hd, const void* q,
-                           const void* k, const void* v, const void* o, const void* d_o, void* dq, void* dk, void* dv,
-                           int64_t sb, int64_t sh, int64_t ss, int64_t osb, int64_t osh, int64_t oss,
-                           const float* lse, float* delta, const void* bias, int64_t bias_sh, int64_t bias_sr,
-                           float scale) {
+static int attn_bwd_entry(void* stream, int dtype, int64_t B, int64_t nh, int64_t S, int64_t hd, const void* q,
+                          const void* k, const void* v, const void* o, const void* d_o, void* dq, void* dk, void* dv,
+                          int64_t sb, int64_t sh, int64_t ss, int64_t osb, int64_t osh, int64_t oss, const float* lse,
+                          float* delta, const void* bias, int64_t bias_sh, int64_t bias_sr, const void* slopes,
+                          float scale) {
   if (!q || !k || !v || !o || !d_o || !dq || !dk || !dv || !lse || !delta) return TF_EINVAL;
   const int rc = attn_check(dtype, B, nh, S, hd, sb, sh, ss, osb, osh, oss, bias, bias_sh, bias_sr);
   if (rc != TF_OK) return rc;
@@ -921,12 +956,46 @@ extern "C" int tf_attn_bwd(void* stream, int dtype, int64_t B, int64_t nh, int64
   if (bias && (reinterpret_cast<uintptr_t>(bias) & 15)) return TF_EALIGN;
   AttnParams p = {};
   p.q = q; p.k = k; p.v = v; p.o = o; p.d_o = d_o; p.dq = dq; p.dk = dk; p.dv = dv;
-  p.lse = const_cast<float*>(lse); p.delta = delta; p.bias = bias;
+  p.lse = const_cast<float*>(lse); p.delta = delta; p.bias = bias; p.slopes = slopes;
   p.sb = sb; p.sh = sh; p.ss = ss; p.osb = osb; p.osh = osh; p.oss = oss;
   p.bias_sh = bias_sh; p.bias_sr = bias_sr;
   p.B = (int)B; p.nh = (int)nh; p.S = (int)S;
   p.scale = scale; p.scale_log2 = scale * kLog2e;
   hipStream_t st = (hipStream_t)stream;
-  if (dtype == TF_F16) return attn_dispatch<f16, false>(st, (int)hd, bias != nullptr, p);
-  return attn_dispatch<bf16, false>(st, (int)hd, bias != nullptr, p);
+  if (dtype == TF_F16) return attn_dispatch<f16, false>(st, (int)hd, p);
+  return attn_dispatch<bf16, false>(st, (int)hd, p);
+}
+
+extern "C" int tf_attn_fwd(void* stream, int dtype, int64_t B, int64_t nh, int64_t S, int64_t hd, const void* q,
+                           const void* k, const void* v, void* o, int64_t sb, int64_t sh, int64_t ss, int64_t osb,
+                           int64_t osh, int64_t oss, float* lse, const void* bias, int64_t bias_sh, int64_t bias_sr,
+                           float scale) {
+  return attn_fwd_entry(stream, dtype, B, nh, S, hd, q, k, v, o, sb, sh, ss, osb, osh, oss, lse, bias, bias_sh, bias_sr,
+                        nullptr, scale);
+}
+
+extern "C" int tf_attn_bwd(void* stream, int dtype, int64_t B, int64_t nh, int64_t S, int64_t hd, const void* q,
+                           const void* k, const void* v, const void* o, const void* d_o, void* dq, void* dk, void* dv,
+                           int64_t sb, int64_t sh, int64_t ss, int64_t osb, int64_t osh, int64_t oss,
+                           const float* lse, float* delta, const void* bias, int64_t bias_sh, int64_t bias_sr,
+                           float scale) {
+  return attn_bwd_entry(stream, dtype, B, nh, S, hd, q, k, v, o, d_o, dq, dk, dv, sb, sh, ss, osb, osh, oss, lse, delta,
+                        bias, bias_sh, bias_sr, nullptr, scale);
+}
+
+extern "C" int tf_attn_alibi_fwd(void* stream, int dtype, int64_t B, int64_t nh, int64_t S, int64_t hd, const void* q,
+                                 const void* k, const void* v, void* o, int64_t sb, int64_t sh, int64_t ss,
+                                 int64_t osb, int64_t osh, int64_t oss, float* lse, const void* slopes, float scale) {
+  if (!slopes || (reinterpret_cast<uintptr_t>(slopes) & 1)) return TF_EINVAL;
+  return attn_fwd_entry(stream, dtype, B, nh, S, hd, q, k, v, o, sb, sh, ss, osb, osh, oss, lse, nullptr, 0, 0, slopes,
+                        scale);
+}
+
+extern "C" int tf_attn_alibi_bwd(void* stream, int dtype, int64_t B, int64_t nh, int64_t S, int64_t hd, const void* q,
+                                 const void* k, const void* v, const void* o, const void* d_o, void* dq, void* dk,
+                                 void* dv, int64_t sb, int64_t sh, int64_t ss, int64_t osb, int64_t osh, int64_t oss,
+                                 const float* lse, float* delta, const void* slopes, float scale) {
+  if (!slopes || (reinterpret_cast<uintptr_t>(slopes) & 1)) return TF_EINVAL;
+  return attn_bwd_entry(stream, dtype, B, nh, S, hd, q, k, v, o, d_o, dq, dk, dv, sb, sh, ss, osb, osh, oss, lse, delta,
+                        nullptr, 0, 0, slopes, scale);
 }

@@ -273,7 +273,11 @@ def _check_attn(q, k, v, bias):
     if not (q.dtype == k.dtype == v.dtype) or q.dtype not in (torch.float16, torch.bfloat16):
         raise TypeError("q, k, v must share one 16-bit dtype")
     require_cuda(q, k, v, bias)
-    if bias is not None:
+    if bias is not None and bias.ndim == 1:
+        # ALiBi in closed form: the nh slopes as the reference rounds them (fp16, transformer.py:68)
+        if bias.shape[0] != nh or bias.dtype != torch.float16:
+            raise ValueError("ALiBi slopes must be a (nh,) float16 vector")
+    elif bias is not None:
         # kernels/biased_attention.py:199-207 of the reference
         if bias.ndim != 3 or bias.shape[0] != nh:
             raise ValueError("attention bias must be (nh, S', S')")
@@ -300,7 +304,9 @@ def _strided_ok(t):
 
 
 def flash_wrapper_fwd(q, k, v, bias=None, out=None):
-    """Causal attention forward -> (out, lse).  ``out`` has q's strides unless a
+    """Causal attention forward -> (out, lse).  ``bias``: None, a dense (nh, S', S') matrix, or
+    the (nh,) float16 ALiBi slopes (the bias -slope_h * (i - j) is then computed in the kernel
+    with the roundings of the reference's dense matrix).  ``out`` has q's strides unless a
     (B, nh, S, hd) view is passed in; ``lse`` is (B, nh, S) fp32 in the log2
     domain (the reference keeps fp16 m and l, kernels/attention.py:171-217 and
     kernels/biased_attention.py:188-245)."""
@@ -312,6 +318,13 @@ def flash_wrapper_fwd(q, k, v, bias=None, out=None):
     elif out.shape != q.shape or out.dtype != q.dtype or not _strided_ok(out):
         raise ValueError("attention output buffer must match q in shape and dtype, with aligned strides")
     lse = torch.empty((b, nh, s), dtype=torch.float32, device=q.device)
+    if bias is not None and bias.ndim == 1:
+        slopes = bias.contiguous()
+        check(load().tf_attn_alibi_fwd(stream_ptr(), dtype_code(q.dtype), b, nh, s, hd, q.data_ptr(), k.data_ptr(),
+                                       v.data_ptr(), out.data_ptr(), q.stride(0), q.stride(1), q.stride(2),
+                                       out.stride(0), out.stride(1), out.stride(2), lse.data_ptr(), slopes.data_ptr(),
+                                       1.0 / math.sqrt(hd)))
+        return out, lse
     bias, bptr, bsh, bsr = _bias_args(bias)
     check(load().tf_attn_fwd(stream_ptr(), dtype_code(q.dtype), b, nh, s, hd, q.data_ptr(), k.data_ptr(),
                              v.data_ptr(), out.data_ptr(), q.stride(0), q.stride(1), q.stride(2), out.stride(0),
@@ -338,6 +351,14 @@ def flash_wrapper_bwd(grad_out, out, q, k, v, lse, bias=None, grads=None):
     if any(t.stride() != q.stride() or t.data_ptr() % 16 for t in grads):
         raise ValueError("attention gradient buffers must share q's strides")
     delta = torch.empty((b, nh, s), dtype=torch.float32, device=q.device)
+    if bias is not None and bias.ndim == 1:
+        slopes = bias.contiguous()
+        check(load().tf_attn_alibi_bwd(stream_ptr(), dtype_code(q.dtype), b, nh, s, hd, q.data_ptr(), k.data_ptr(),
+                                       v.data_ptr(), out.data_ptr(), grad_out.data_ptr(), dq.data_ptr(), dk.data_ptr(),
+                                       dv.data_ptr(), q.stride(0), q.stride(1), q.stride(2), out.stride(0),
+                                       out.stride(1), out.stride(2), lse.data_ptr(), delta.data_ptr(),
+                                       slopes.data_ptr(), 1.0 / math.sqrt(hd)))
+        return dq, dk, dv
     bias, bptr, bsh, bsr = _bias_args(bias)
     check(load().tf_attn_bwd(stream_ptr(), dtype_code(q.dtype), b, nh, s, hd, q.data_ptr(), k.data_ptr(),
                              v.data_ptr(), out.data_ptr(), grad_out.data_ptr(), dq.data_ptr(), dk.data_ptr(),

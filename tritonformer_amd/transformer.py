@@ -90,6 +90,11 @@ FUSE_ADD_LN = True
 # one kernel, and the table gradients a chain-ordered scatter-add; False: two nn.Embedding
 # calls and an addition as in the reference (transformer.py:311-323).
 FUSE_EMBED = True
+# True (read when a model with attn_bias=True is built): no dense (nh, S, S) ALiBi matrix --
+# 805 MB at 24 heads x 4096 -- is made; the attention kernels compute -slope_h * (i - j) from
+# the nh slopes with the roundings of that matrix, bit-identical results.  False: the dense
+# buffer "attn_bias" as in the reference (transformer.py:296-302).
+FUSE_ALIBI = True
 
 
 def _weights_init(model: nn.Module, num_layers: int) -> None:
@@ -221,14 +226,29 @@ class Transformer(nn.Module):
         self.logits_out = tnn.Linear(config.hidden_size, config.vocab_size, bias=False, device=device,
                                      dtype=param_dtype, fuse_activation=False)
         _weights_init(self, config.num_hidden_layers)
-        if config.attn_bias:
+        if config.attn_bias and FUSE_ALIBI:
+            # the kernels rebuild the bias from the slopes; a checkpoint's dense "attn_bias" entry
+            # is dropped on load and regenerated on save, so state dicts stay interchangeable
+            self.attn_bias = None
+            self.register_buffer("alibi_slopes", torch.tensor(get_slopes(config.num_attention_heads), device=device,
+                                                              dtype=torch.float16), persistent=False)
+            self._register_load_state_dict_pre_hook(lambda state, prefix, *_: state.pop(prefix + "attn_bias", None))
+
+            def add_dense_bias(module, state, prefix, _metadata):
+                # a saved state dict still holds the reference's buffer, built when it is asked for
+                state[prefix + "attn_bias"] = generate_alibi_mask(
+                    config.max_position_embeddings, config.num_attention_heads, device=module.alibi_slopes.device)[0]
+
+            self._register_state_dict_hook(add_dense_bias)
+        elif config.attn_bias:
+            self.alibi_slopes = None
             # the bias is an activation-side tensor: always 16-bit, like the reference's
             self.register_buffer(
                 "attn_bias",
                 generate_alibi_mask(config.max_position_embeddings, config.num_attention_heads, device=device)[0],
             )
         else:
-            self.attn_bias = None
+            self.attn_bias = self.alibi_slopes = None
 
     def forward(self, input_ids: torch.Tensor, labels: Optional[torch.Tensor]):
         batch_size, seq_len = input_ids.shape
@@ -249,6 +269,8 @@ class Transformer(nn.Module):
                 hidden_states = hidden_states.to(amp_dtype)
         if amp_dtype is not None and attn_bias is not None:
             attn_bias = attn_bias.to(amp_dtype)
+        if self.alibi_slopes is not None:
+            attn_bias = self.alibi_slopes
         if FUSE_ADD_LN and len(self.layer_list) > 0:
             pending = None
             for layer in self.layer_list:
