@@ -187,6 +187,41 @@ def mfma_probe(dtype, device, iters=20000):
     return out
 
 
+def attention_probe(workload, dtype, device, iters=20):
+    """The attention kernels of one layer of ``workload`` alone (forward, delta, dK/dV, dQ on the
+    packed projection layout the model uses), ``iters`` times: what `rocprofv3 --pmc` is pointed at
+    for their counters.  Returns the average time of one forward + backward."""
+    import tritonformer_amd as T
+
+    L, d, nh, hd, f, S, B, lin_bias, alibi = WORKLOADS[workload]
+    gen = torch.Generator(device="cpu").manual_seed(0)
+    qkv = torch.randn(B, S, 3, nh, hd, generator=gen).to(dtype).to(device).requires_grad_(True)
+    grad = torch.randn(B, S, nh * hd, generator=gen).to(dtype).to(device)
+    bias = None
+    if alibi:
+        from tritonformer_amd.transformer import get_slopes
+        bias = torch.tensor(get_slopes(nh), dtype=torch.float16, device=device)
+
+    def once():
+        qkv.grad = None
+        T.fast_causal_attention_qkvpacked.apply(qkv, bias).backward(grad)
+
+    for _ in range(3):
+        once()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        once()
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) / iters * 1e3
+    flop = 7.0 * B * S * S * nh * hd  # causal: 2 forward + 5 backward matrix products at half cost
+    return {"probe": "attention forward + backward of one layer", "workload": workload,
+            "dtype": str(dtype).replace("torch.", ""), "iters": iters, "us_per_layer": round(us, 1),
+            "tflops": round(flop / us / 1e6, 1)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -202,6 +237,8 @@ def main():
     ap.add_argument("--mfma-probe", action="store_true",
                     help="instead of the step: sustained rate of the GEMM kernel's MFMA stream alone (no memory "
                          "traffic) for constant and for random operand values, one JSON line")
+    ap.add_argument("--attention-probe", action="store_true",
+                    help="instead of the step: the attention kernels of one layer of the workload alone, one JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported "
@@ -213,6 +250,9 @@ def main():
     device = torch.device("cuda:0")
     if args.mfma_probe:
         print(json.dumps(mfma_probe(dtype, device)))
+        return
+    if args.attention_probe:
+        print(json.dumps(attention_probe(args.workload, dtype, device)))
         return
     L, d, nh, hd, f, S, B, lin_bias, alibi = WORKLOADS[args.workload]
     model, tokens = make_model(args.workload, device, dtype)
