@@ -265,6 +265,22 @@ int tf_embedding_bwd(void* stream, int grad_dtype, int param_dtype, int64_t T, i
                      void* d_tok, int64_t ld_dtok, void* d_pos, int64_t ld_dpos,
                      void* workspace, int64_t workspace_bytes);
 
+/* One AdamW step (decoupled weight decay, no amsgrad; the arithmetic of torch.optim.AdamW
+ * operation for operation) over `count` fp32 parameter tensors in as few launches as their
+ * descriptors fit into: p, m, v updated in place from the fp32 gradient; when `shadow` is
+ * set, the updated parameter is also written there rounded to shadow_dtype -- the 16-bit
+ * operand the next forward pass would otherwise produce with a cast kernel.  `step` counts
+ * from 1.  No counterpart in the reference, which ships no optimizer; it is what turns the
+ * forward + backward step that the reference times (README.md:62-77) into a training
+ * step.  `tensors`: HOST array. */
+typedef struct tf_adamw_tensor {
+  void* param; const void* grad; void* exp_avg; void* exp_avg_sq;   /* fp32, `count` elements each */
+  void* shadow;                                                      /* 16-bit, or null */
+  int64_t count;
+} tf_adamw_tensor;
+int tf_adamw_step(void* stream, int shadow_dtype, int count, const tf_adamw_tensor* tensors,
+                  float lr, float beta1, float beta2, float eps, float weight_decay, int64_t step);
+
 /* Row softmax / its backward dx = y * (dy - sum(y*dy)); dtype f16/bf16/f32.
  * Replaces softmax_fwd / softmax_bwd (kernels/softmax.py:37-54, 95-111); the
  * backward writes a new buffer instead of overwriting grad_out. */

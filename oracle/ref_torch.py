@@ -20,6 +20,8 @@ Pinning status (which independent check fixes each function):
   get_slopes / alibi mask   closed forms for n = 8, 16, 24
   embedding / _bwd          element loops on a tiny case (tests/test_oracle.py); F.embedding and
                             its autograd; one-hot matrix product
+  adamw_step                torch.optim.AdamW on the CPU over several steps; closed form of the
+                            first step (p - lr*wd*p - lr*sign(g) up to eps)
   RefTransformer            zero-initialised LM head -> loss = ln(vocab) exactly and zero grads
                             upstream; parameter-name list; committed config-1 fixture
 No function of this oracle is "parity unpinned".
@@ -136,6 +138,18 @@ def embedding_bwd(ids, g, vocab: int, positions: Optional[int] = None):
     d_pos = torch.zeros((positions, g.shape[-1]), dtype=torch.float32)
     d_pos[:s] = g.sum(0)
     return d_tok, d_pos
+
+
+def adamw_step(p, g, m, v, step: int, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=1e-2):
+    """One AdamW step (decoupled weight decay, no amsgrad) on fp32 tensors, out of place:
+    returns (p, m, v) after the step; ``step`` counts from 1."""
+    b1, b2 = betas
+    p = p * (1.0 - lr * weight_decay)
+    m = m + (g - m) * (1.0 - b1)
+    v = v * b2 + (1.0 - b2) * g * g
+    bc1, bc2 = 1.0 - b1 ** step, 1.0 - b2 ** step
+    denom = v.sqrt() / math.sqrt(bc2) + eps
+    return p - (lr / bc1) * (m / denom), m, v
 
 
 def get_slopes(n: int) -> List[float]:

@@ -124,6 +124,25 @@ def test_embedding_rejects_bad_arguments():
     assert bwd(gd=0, pd=1) == -2
 
 
+def test_adamw_rejects_bad_arguments():
+    import ctypes
+
+    lib = _lib.load()
+
+    def call(count=1, step=1, beta1=0.9, lr=1e-3, shadow=None, shadow_dtype=0, grad=FAKE, param=FAKE):
+        arr = (_lib.AdamTensor * 1)()
+        arr[0].param, arr[0].grad, arr[0].exp_avg, arr[0].exp_avg_sq = param, grad, FAKE, FAKE
+        arr[0].shadow, arr[0].count = shadow, 16
+        return lib.tf_adamw_step(None, shadow_dtype, count, ctypes.cast(arr, ctypes.c_void_p), lr, beta1, 0.999, 1e-8,
+                                 0.01, step)
+
+    assert call(step=0) == -1 and call(beta1=1.0) == -1 and call(lr=-1.0) == -1 and call(grad=None) == -1
+    assert call(param=0x1002) == -3            # fp32 tensors are 4-byte aligned
+    assert call(shadow=FAKE, shadow_dtype=2) == -2   # a 16-bit type for the copies
+    assert lib.tf_adamw_step(None, 0, 1, None, 1e-3, 0.9, 0.999, 1e-8, 0.01, 1) == -1
+    assert lib.tf_adamw_step(None, 0, 0, None, 1e-3, 0.9, 0.999, 1e-8, 0.01, 1) == 0   # nothing to do
+
+
 def test_attention_rejects_bad_shapes():
     lib = _lib.load()
 

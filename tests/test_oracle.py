@@ -211,6 +211,26 @@ def test_embedding_vs_loops_and_library():
     assert torch.allclose(onehot.T @ g.reshape(b * s, d), d_tok, atol=1e-6)
 
 
+def test_adamw_vs_library_and_first_step_closed_form():
+    torch.manual_seed(5)
+    p0 = torch.randn(37, 11)
+    hyper = dict(lr=3e-3, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+    lib_p = p0.clone().requires_grad_(True)
+    opt = torch.optim.AdamW([lib_p], **hyper)
+    p, m, v = p0.clone(), torch.zeros_like(p0), torch.zeros_like(p0)
+    for step in range(1, 6):
+        g = torch.randn_like(p0) * (0.1 * step)
+        lib_p.grad = g.clone()
+        opt.step()
+        p, m, v = R.adamw_step(p, g, m, v, step, **hyper)
+        assert torch.allclose(p, lib_p.detach(), rtol=1e-6, atol=1e-7), step
+        if step == 1:  # m / sqrt(v) = sign(g) after bias correction: p1 = p0 (1 - lr wd) - lr sign(g)
+            want = p0 * (1 - hyper["lr"] * hyper["weight_decay"]) - hyper["lr"] * torch.sign(g)
+            assert torch.allclose(p, want, rtol=1e-5, atol=1e-6)
+    st = opt.state[lib_p]
+    assert torch.allclose(m, st["exp_avg"], rtol=1e-6, atol=1e-8) and torch.allclose(v, st["exp_avg_sq"], rtol=1e-6, atol=1e-10)
+
+
 def test_model_known_answers():
     cfg = R.RefConfig(50304, 64, 32, 2, 32, 128, 2, True, False)
     torch.manual_seed(0)

@@ -30,6 +30,7 @@ SIGNATURES = {
     "tf_embedding_fwd": (_i, [_vp, _i, _i, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _i64, _vp, _i64]),
     "tf_embedding_bwd_workspace_bytes": (_i64, [_i64]),
     "tf_embedding_bwd": (_i, [_vp, _i, _i, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64]),
+    "tf_adamw_step": (_i, [_vp, _i, _i, _vp, _f, _f, _f, _f, _f, _i64]),
     "tf_probe_mfma_rate": (_i, [_vp, _i, _vp, _i, _vp]),
     "tf_probe_mfma_rate_flops": (_i64, [_i]),
     "tf_gemm_group": (_i, [_vp, _i, _i, _i, _i, _i, _vp, _vp, _i64]),
@@ -61,6 +62,12 @@ SIGNATURES = {
     "tf_colsum_partial_bytes": (_i64, [_i64, _i64]),
     "tf_relu_mask": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64]),
 }
+
+class AdamTensor(ctypes.Structure):
+    """tf_adamw_tensor of the C header."""
+    _fields_ = [("param", ctypes.c_void_p), ("grad", ctypes.c_void_p), ("exp_avg", ctypes.c_void_p),
+                ("exp_avg_sq", ctypes.c_void_p), ("shadow", ctypes.c_void_p), ("count", ctypes.c_int64)]
+
 
 class GemmProblem(ctypes.Structure):
     """`tf_gemm_problem` of include/tritonformer_amd.h."""
