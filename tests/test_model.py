@@ -81,6 +81,55 @@ def test_fresh_model_known_answers(dev):
     assert model(ids, None).shape == (2, 128, 50304)          # labels=None returns the logits only
 
 
+# the four GPU configurations of the baseline at their full size:
+# (layers, d, heads, head_dim, ffn, seq, batch, linear_bias, alibi, autocast dtype)
+FULL_SIZE = {
+    "160M ctx2048 bs8, linear bias": (12, 768, 12, 64, 3072, 2048, 8, True, False, torch.float16),
+    "410M ctx2048 bs4 (headline)": (24, 1024, 16, 64, 4096, 2048, 4, False, False, torch.float16),
+    "840M ALiBi ctx4096 bs1": (24, 1536, 24, 64, 6144, 4096, 1, False, True, torch.float16),
+    "1.4B hd128 ctx2048 bs2, bf16": (24, 2048, 16, 128, 8192, 2048, 2, False, False, torch.bfloat16),
+}
+
+
+@pytest.mark.parametrize("name", list(FULL_SIZE))
+def test_full_size_configurations_known_answers(name, dev):
+    """Size-independent properties at the baseline's real shapes, fp32 master weights under
+    autocast: with the reference's initialisation (LM head zero, transformer.py:104-105) the
+    loss is ln(50304) whatever the rest of the network computes, and the loss gradient
+    reaches the LM head only; with a random LM head two steps give the same bits, every
+    parameter gets a finite gradient and the loss is ln(50304) + d * 0.02^2 / 2 (Gaussian logits
+    of variance d * 0.02^2 over a unit-variance LayerNorm output)."""
+    layers, d, nh, hd, f, seq, batch, lin_bias, alibi, dtype = FULL_SIZE[name]
+    cfg = TransformerConfig(50304, d, seq, nh, hd, f, layers, lin_bias, alibi)
+    torch.manual_seed(0)
+    model = Transformer(cfg, device=dev, param_dtype=torch.float32)
+    ids = torch.randint(0, 50304, (batch, seq), device=dev)
+    with torch.autocast("cuda", dtype=dtype):
+        _, loss = model(ids, ids)
+    assert abs(loss.item() - math.log(50304)) < (1e-2 if dtype == torch.float16 else 4e-2)
+    (loss * LOSS_SCALE).backward()
+    for pname, p in model.named_parameters():
+        if pname.startswith("logits_out"):
+            assert p.grad.abs().max() > 0
+        else:
+            assert p.grad is None or p.grad.abs().max() == 0, pname
+    model.logits_out.weight.data.normal_(0.0, 0.02)
+    runs = []
+    for _ in range(2):
+        model.zero_grad(set_to_none=True)
+        with torch.autocast("cuda", dtype=dtype):
+            _, loss = model(ids, ids)
+        (loss * LOSS_SCALE).backward()
+        runs.append((loss.item(), model.layer_list[0].attention.q_proj.weight.grad.clone(),
+                     model.embed_tokens.weight.grad.clone()))
+    assert runs[0][0] == runs[1][0] and torch.equal(runs[0][1], runs[1][1]) and torch.equal(runs[0][2], runs[1][2])
+    # LayerNorm output has unit variance, so the logits are ~ N(0, d * 0.02^2) and independent of the
+    # label: E[loss] = ln V + d * 0.02^2 / 2
+    assert abs(runs[0][0] - (math.log(50304) + 0.5 * d * 0.02 ** 2)) < 0.05
+    for pname, p in model.named_parameters():
+        assert p.grad is not None and torch.isfinite(p.grad).all() and p.grad.abs().max() > 0, pname
+
+
 def test_alibi_model(dev):
     """attn_bias=True: no position embedding, dense ALiBi mask larger than the sequence."""
     cfg = R.RefConfig(50304, 256, 192, 4, 64, 512, 2, False, True)
