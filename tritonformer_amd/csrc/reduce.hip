@@ -59,14 +59,32 @@ __global__ __launch_bounds__(256) void colsum_partial(int64_t rows, int cols, co
   }
 }
 
+// Second stage: out[c] = sum over groups of partial[g][c], in a fixed order.  A workgroup takes 32
+// columns; its 8 slices of 32 lanes each add up every 8th group (independent loads in flight
+// instead of one dependent chain per column), then the slices are combined through LDS.
 template <typename T>
 __global__ __launch_bounds__(256) void colsum_final(int groups, int cols, const float* __restrict__ partial,
                                                      T* __restrict__ out) {
-  const int c = blockIdx.x * 256 + threadIdx.x;
-  if (c >= cols) return;
-  float s = 0.f;
-  for (int g = 0; g < groups; ++g) s += partial[(int64_t)g * cols + c];
-  out[c] = (T)s;
+  __shared__ float red[8][32];
+  const int lane32 = threadIdx.x & 31, slice = threadIdx.x >> 5;
+  const int c = blockIdx.x * 32 + lane32;
+  float s0 = 0.f, s1 = 0.f;
+  if (c < cols) {
+    int g = slice;
+    for (; g + 8 < groups; g += 16) {
+      s0 += partial[(int64_t)g * cols + c];
+      s1 += partial[(int64_t)(g + 8) * cols + c];
+    }
+    if (g < groups) s0 += partial[(int64_t)g * cols + c];
+  }
+  red[slice][lane32] = s0 + s1;
+  __syncthreads();
+  if (slice == 0 && c < cols) {
+    float s = 0.f;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) s += red[k][lane32];
+    out[c] = (T)s;
+  }
 }
 
 template <typename T, bool VEC>
@@ -107,7 +125,7 @@ static int colsum_launch(hipStream_t st, int64_t rows, int64_t cols, const void*
   else
     colsum_partial<T, false><<<grid, block, 0, st>>>(rows, (int)cols, (const T*)x, ldx, partial, rpg);
   TF_CHECK_LAUNCH();
-  colsum_final<T><<<dim3(ceil_div(cols, 256)), block, 0, st>>>(groups, (int)cols, partial, (T*)out);
+  colsum_final<T><<<dim3(ceil_div(cols, 32)), block, 0, st>>>(groups, (int)cols, partial, (T*)out);
   TF_CHECK_LAUNCH();
   return TF_OK;
 }
