@@ -188,7 +188,7 @@ def mfma_probe(dtype, device, iters=20000):
 
 
 def attention_probe(workload, dtype, device, iters=20):
-    """The attention kernels of one layer of ``workload`` alone (forward, delta, dK/dV, dQ on the
+    """The attention kernels of one layer of ``workload`` alone (forward, dQ, dK/dV on the
     packed projection layout the model uses), ``iters`` times: what `rocprofv3 --pmc` is pointed at
     for their counters.  Returns the average time of one forward + backward."""
     import tritonformer_amd as T

@@ -29,7 +29,7 @@ struct AttnParams {
   const void *q, *k, *v, *o, *d_o;
   void *out, *dq, *dk, *dv;
   float* lse;    // written by fwd, read by bwd
-  float* delta;  // written by the bwd pre-pass
+  float* delta;  // -rowsum(dO * O): written by the dQ pass, read by the dK/dV pass
   const void* bias;
   const void* slopes;         // ALiBi in closed form: nh fp16 slopes instead of a dense bias
   int64_t sb, sh, ss;         // element strides of q, k, v and of dq, dk, dv
@@ -394,30 +394,6 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (BMODE == kDenseBias ? 2 : 3)) v
 }
 
 // ===========================================================================
-// Backward pre-pass: delta[b,h,q] = -sum_d dO[q,d] * O[q,d] (stored negated).
-// ===========================================================================
-template <typename T, int HD>
-__global__ __launch_bounds__(256) void attn_delta_kernel(AttnParams p) {
-  constexpr int LPR = HD / 8;       // lanes per row
-  constexpr int RPB = 256 / LPR;    // rows per workgroup
-  const int nbh = p.B * p.nh;
-  const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / LPR;  // over nbh * S
-  if (row >= (int64_t)nbh * p.S) return;
-  const int bh = (int)(row / p.S), s = (int)(row % p.S);
-  const int64_t off = (int64_t)(bh / p.nh) * p.osb + (int64_t)(bh % p.nh) * p.osh + (int64_t)s * p.oss +
-                      (threadIdx.x % LPR) * 8;
-  float a[8], g[8];
-  Chunk<T>::load((const T*)p.o + off, a);
-  Chunk<T>::load((const T*)p.d_o + off, g);
-  float acc = 0.f;
-#pragma unroll
-  for (int e = 0; e < 8; ++e) acc += a[e] * g[e];
-#pragma unroll
-  for (int o = LPR / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
-  if (threadIdx.x % LPR == 0) p.delta[row] = -acc;  // negated: both consumers start dP from -delta
-}
-
-// ===========================================================================
 // dK/dV pass.  Workgroup: 4 waves x 32 keys; query blocks of 64 from the
 // diagonal downwards.  Q and dO tiles (+ their lse / delta) go through LDS.
 // ===========================================================================
@@ -698,7 +674,21 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (BMODE != kNoBias ? 2 : 3)) void
   }
   if (active) {
     neg_lse = -p.lse[(int64_t)bh * p.S + myq];
-    neg_delta = p.delta[(int64_t)bh * p.S + myq];  // the pre-pass stores it negated
+    // -delta = -rowsum(dO * O) of this lane's query row: each of the two lanes that share a row has half
+    // of it.  Stored for the dK/dV pass, which runs after this one.
+    const T* Orow = (const T*)p.o + (int64_t)b * p.osb + (int64_t)h * p.osh + (int64_t)myq * p.oss + (lane >> 5) * 8;
+    float half_sum = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const v8 o = __builtin_bit_cast(v8, ld16(Orow + ks * 16));
+#pragma unroll
+      for (int e = 0; e < 8; ++e) half_sum = fmaf((float)o[e], (float)dof[ks][e], half_sum);
+    }
+    const unsigned u = __builtin_bit_cast(unsigned, half_sum);
+    const auto both = __builtin_amdgcn_permlane32_swap(u, u, false, false);  // own half and the partner's
+    const unsigned u0 = both[0], u1 = both[1];
+    neg_delta = -(__builtin_bit_cast(float, u0) + __builtin_bit_cast(float, u1));
+    if (lane < 32) p.delta[(int64_t)bh * p.S + myq] = neg_delta;
   }
   f32x16 dq[DT];
 #pragma unroll
@@ -862,24 +852,21 @@ static int fwd_launch(hipStream_t st, const AttnParams& p) {
   return TF_OK;
 }
 
+// dQ pass first: it also produces the -delta rows that the dK/dV pass reads.
 template <typename T, int HD, int MODE>
 static int bwd_launch(hipStream_t st, const AttnParams& p) {
-  const int64_t rows = (int64_t)p.B * p.nh * p.S;
-  constexpr int rpb = 256 / (HD / 8);
-  attn_delta_kernel<T, HD><<<dim3((unsigned)((rows + rpb - 1) / rpb)), dim3(256), 0, st>>>(p);
-  TF_CHECK_LAUNCH();
   const unsigned grid = (unsigned)(((p.S + 127) / 128) * p.B * p.nh);
   {
-    constexpr int lds = 2 * (2 * SeqTile<T, 64, HD>::BYTES + 2 * 64 * 4 + (MODE == kDenseBias ? 64 * 128 * 2 : 0));
-    auto kernel = attn_dkdv_kernel<T, HD, MODE>;
+    constexpr int lds = 2 * (2 * SeqTile<T, 64, HD>::BYTES + (MODE == kDenseBias ? BiasTile::BYTES : 0));
+    auto kernel = attn_dq_kernel<T, HD, MODE>;
     static bool once = (allow_lds(kernel, lds), true);
     (void)once;
     kernel<<<dim3(grid), dim3(256), lds, st>>>(p);
     TF_CHECK_LAUNCH();
   }
   {
-    constexpr int lds = 2 * (2 * SeqTile<T, 64, HD>::BYTES + (MODE == kDenseBias ? BiasTile::BYTES : 0));
-    auto kernel = attn_dq_kernel<T, HD, MODE>;
+    constexpr int lds = 2 * (2 * SeqTile<T, 64, HD>::BYTES + 2 * 64 * 4 + (MODE == kDenseBias ? 64 * 128 * 2 : 0));
+    auto kernel = attn_dkdv_kernel<T, HD, MODE>;
     static bool once = (allow_lds(kernel, lds), true);
     (void)once;
     kernel<<<dim3(grid), dim3(256), lds, st>>>(p);
