@@ -34,7 +34,8 @@ def amp_fwd(fwd=None, *, keep=()):
         ctx._fwd_used_autocast = False
         # dtypes the caller passed in, before any autocast cast (fp32 master weights)
         ctx.arg_dtypes = tuple(a.dtype if isinstance(a, torch.Tensor) else None for a in args)
-        if torch.is_autocast_enabled("cuda"):
+        ctx.amp_active = torch.is_autocast_enabled("cuda")  # for bodies that cast their `keep` arguments themselves
+        if ctx.amp_active:
             dtype = torch.bfloat16 if ctx._dtype == torch.bfloat16 else torch.float16
             with torch.autocast(device_type="cuda", enabled=False):
                 cast = tuple(a if i in keep else _cast(a, dtype) for i, a in enumerate(args))

@@ -118,22 +118,25 @@ class AttentionBlock(Function):
         attn_bias = _bias_for(attn_bias, x.dtype)
         b, s, d = x.shape
         hd = d // num_heads
-        w_qkv = cast_pack([wq, wk, wv], x.dtype)
-        w_o = cast_pack([wo], x.dtype)
+        # the four (d, d) weights side by side in one 16-bit (d, 4d) matrix, one conversion kernel;
+        # the GEMMs take its first three column blocks and its last one as strided operands
+        packed = cast_pack([wq, wk, wv, wo], x.dtype)
+        w_qkv, w_o = packed[:, : 3 * d], packed[:, 3 * d:]
         qkv = mm(x, w_qkv).view(b, s, 3, num_heads, hd)
         q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
         attn = torch.empty((b, s, num_heads, hd), dtype=x.dtype, device=x.device)
         _, lse = flash_wrapper_fwd(q, k, v, attn_bias, out=attn.permute(0, 2, 1, 3))
         attn = attn.view(b, s, d)
-        ctx.save_for_backward(x, w_qkv, w_o, qkv, attn, lse, attn_bias)
+        ctx.save_for_backward(x, packed, qkv, attn, lse, attn_bias)
         ctx.weight_dtype = wq.dtype
         return mm(attn, w_o)
 
     @staticmethod
     @amp_bwd
     def backward(ctx: Any, grad_output: torch.Tensor):
-        x, w_qkv, w_o, qkv, attn, lse, attn_bias = ctx.saved_tensors
+        x, packed, qkv, attn, lse, attn_bias = ctx.saved_tensors
         b, s, _, nh, hd = qkv.shape
+        w_qkv, w_o = packed[:, : 3 * nh * hd], packed[:, 3 * nh * hd:]
         d_attn = mm(grad_output, w_o.T).view(b, s, nh, hd).permute(0, 2, 1, 3)
         q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
         dqkv = torch.empty_like(qkv)

@@ -9,6 +9,8 @@ from .kernels import cast_pack, gemm, mask_grad, mm, mm_dw, mm_dw_group, unbroad
 
 # True: weight gradients that are available together are computed by one grouped launch
 GROUP_DW = True
+# True: fp32 master weights of one block are converted to 16 bits by one kernel launch, not one each
+PACK_CASTS = True
 
 
 def _grads(ctx, grad_output, inputs, weights):
@@ -107,8 +109,17 @@ class MLPReLU(Function):
     (two Functions and an in-place mask kernel, linear.py:47-102)."""
 
     @staticmethod
-    @amp_fwd
+    @amp_fwd(keep=(1, 3))
     def forward(ctx, input, w1, b1, w2, b2):
+        if ctx.amp_active and (w1.dtype != input.dtype or w2.dtype != input.dtype):
+            # what autocast's cast of the two weights does -- as ONE conversion kernel over both when
+            # they are stored alike (two matrices of d*f elements each seen as two rows)
+            if (PACK_CASTS and w1.dtype == w2.dtype == torch.float32 and w1.numel() == w2.numel()
+                    and w1.is_contiguous() and w2.is_contiguous() and w1.numel() % 8 == 0):
+                both = cast_pack([w1.view(1, -1), w2.view(1, -1)], input.dtype)
+                w1, w2 = both[0, : w1.numel()].view(w1.shape), both[0, w1.numel():].view(w2.shape)
+            else:
+                w1, w2 = w1.to(input.dtype), w2.to(input.dtype)
         hidden = gemm(input, w1, b1, True)
         out = gemm(hidden, w2, b2, False)
         ctx.save_for_backward(input, w1, w2, hidden)
