@@ -672,6 +672,44 @@ __global__ __launch_bounds__(256) void gemm_reduce(int M, int N, int splits, con
   }
 }
 
+// The same second pass for up to kMaxGroup products of one grouped launch at once (blockIdx.y = product;
+// no bias, no ReLU): one launch instead of one per product.
+struct ReduceItem {
+  const float* partial;
+  void* C;
+  int64_t ldc, chunk_skip;
+  int M, N, splits, chunk_n;
+};
+struct ReduceBatch { ReduceItem it[kMaxGroup]; };
+template <typename TO, bool VEC4>
+__global__ __launch_bounds__(256) void gemm_reduce_group(ReduceBatch batch) {
+  const ReduceItem r = batch.it[blockIdx.y];
+  if (r.splits <= 1) return;
+  const int64_t total = (int64_t)r.M * r.N;
+  TO* C = (TO*)r.C;
+  if (VEC4) {
+    const int64_t quads = total >> 2;
+    for (int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x; q < quads; q += (int64_t)gridDim.x * 256) {
+      f32x4 s = *reinterpret_cast<const f32x4*>(r.partial + q * 4);
+      for (int k = 1; k < r.splits; ++k) s += *reinterpret_cast<const f32x4*>(r.partial + (int64_t)k * total + q * 4);
+      const int64_t i = q * 4;
+      const int m = (int)(i / r.N), n = (int)(i - (int64_t)m * r.N);
+      struct alignas(sizeof(TO) * 4) Quad { TO v[4]; };
+      Quad qd;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) qd.v[e] = (TO)s[e];
+      *reinterpret_cast<Quad*>(C + (int64_t)m * r.ldc + n + (int64_t)(n / r.chunk_n) * r.chunk_skip) = qd;
+    }
+  } else {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+      float s = 0.f;
+      for (int k = 0; k < r.splits; ++k) s += r.partial[(int64_t)k * total + i];
+      const int m = (int)(i / r.N), n = (int)(i - (int64_t)m * r.N);
+      C[(int64_t)m * r.ldc + n + (int64_t)(n / r.chunk_n) * r.chunk_skip] = (TO)s;
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------
 // host side: tile choice, contraction split, launch
 // ---------------------------------------------------------------------------
@@ -867,10 +905,28 @@ static int gemm_group_dispatch(hipStream_t st, const GemmGroup& g) {
   (void)once;
   kernel<<<dim3((unsigned)g.first[g.count]), dim3(512), lds, st>>>(g);
   TF_CHECK_LAUNCH();
+  // second pass of the split contractions: all products of the group in one launch
+  ReduceBatch rb = {};
+  bool any = false, v4 = true;
+  int64_t most = 0;
   for (int i = 0; i < g.count; ++i) {
-    const int rc = launch_reduce<T>(st, g.p[i]);
-    if (rc != TF_OK) return rc;
+    const GemmParams& p = g.p[i];
+    rb.it[i] = {p.partial, p.C, p.ldc, p.chunk_skip, p.M, p.N, p.splits, p.chunk_n};
+    if (p.splits <= 1) continue;
+    any = true;
+    v4 = v4 && p.N % 4 == 0 && p.ldc % 4 == 0 && p.chunk_n % 4 == 0 && p.chunk_skip % 4 == 0 &&
+         (reinterpret_cast<uintptr_t>(p.C) & 15) == 0;
+    const int64_t total = (int64_t)p.M * p.N;
+    if (total > most) most = total;
   }
+  if (!any) return TF_OK;
+  int64_t blocks = ((v4 ? most / 4 : most) + 255) / 256;
+  blocks = blocks > 4096 ? 4096 : (blocks < 1 ? 1 : blocks);
+  const dim3 grid((unsigned)blocks, (unsigned)g.count), block(256);
+  const bool f32 = g.p[0].out_f32 != 0;
+  if (f32) { if (v4) gemm_reduce_group<float, true><<<grid, block, 0, st>>>(rb); else gemm_reduce_group<float, false><<<grid, block, 0, st>>>(rb); }
+  else { if (v4) gemm_reduce_group<T, true><<<grid, block, 0, st>>>(rb); else gemm_reduce_group<T, false><<<grid, block, 0, st>>>(rb); }
+  TF_CHECK_LAUNCH();
   return TF_OK;
 }
 
