@@ -96,6 +96,70 @@ __global__ __launch_bounds__(kCeThreads) void ce_fwd(int V, const T* __restrict_
   }
 }
 
+// Forward for rows that fit into the registers of one workgroup (V <= 8 * NCH * kCeThreads): a
+// thread requests all of its NCH 16-byte chunks at once -- NCH loads in flight instead of four --
+// takes the row maximum first and then the sum of exponentials, both from registers.
+template <typename T, int NCH>
+__global__ __launch_bounds__(kCeThreads) void ce_fwd_regs(int V, const T* __restrict__ logits, RowMap map,
+                                                           const int64_t* __restrict__ labels, T* __restrict__ loss,
+                                                           float* __restrict__ lse) {
+  __shared__ float red[2][kCeThreads / 64];
+  const int64_t row = blockIdx.x;
+  const T* xr = logits + map.at(row);
+  const int nchunk = V >> 3;
+  u32x4 raw[NCH];
+#pragma unroll
+  for (int u = 0; u < NCH; ++u) {
+    const int c = threadIdx.x + u * kCeThreads;
+    if (c < nchunk) raw[u] = ld16(xr + c * 8);
+  }
+  float m = -INFINITY;
+#pragma unroll
+  for (int u = 0; u < NCH; ++u) {
+    if (threadIdx.x + u * kCeThreads < nchunk) {
+      float v[8];
+      unpack8<T>(raw[u], v);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) m = fmaxf(m, v[e]);
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) red[0][wave] = m;
+  __syncthreads();
+  m = red[0][0];
+#pragma unroll
+  for (int w = 1; w < kCeThreads / 64; ++w) m = fmaxf(m, red[0][w]);
+  const float m2 = m * kLog2e;
+  float s = 0.f;
+#pragma unroll
+  for (int u = 0; u < NCH; ++u) {
+    if (threadIdx.x + u * kCeThreads < nchunk) {
+      float v[8];
+      unpack8<T>(raw[u], v);
+      float part = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) part += exp2f(v[e] * kLog2e - m2);
+      s += part;
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+  if ((threadIdx.x & 63) == 0) red[1][wave] = s;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float tot = red[1][0];
+#pragma unroll
+    for (int w = 1; w < kCeThreads / 64; ++w) tot += red[1][w];
+    const float l = (m2 + log2f(tot)) * kLn2;  // natural-log logsumexp
+    lse[row] = l;
+    const int64_t lab = labels[row];
+    const float xl = (lab >= 0 && lab < V) ? (float)xr[lab] : 0.f;
+    loss[row] = (T)(l - xl);
+  }
+}
+
 template <typename T, bool VEC>
 __global__ __launch_bounds__(kCeThreads) void ce_bwd(int V, const T* __restrict__ logits, RowMap map,
                                                       const int64_t* __restrict__ labels,
@@ -135,9 +199,17 @@ template <typename T>
 static int ce_fwd_launch(hipStream_t st, int64_t rows, int64_t V, const void* logits, RowMap map,
                          const int64_t* labels, void* loss, float* lse) {
   const dim3 grid((unsigned)rows), block(kCeThreads);
-  if (row_vectorizable<T>(logits, V, map.ld) && map.outer % 8 == 0)
-    ce_fwd<T, true><<<grid, block, 0, st>>>((int)V, (const T*)logits, map, labels, (T*)loss, lse);
-  else
+  if (row_vectorizable<T>(logits, V, map.ld) && map.outer % 8 == 0) {
+    const int64_t per_thread = (V / 8 + kCeThreads - 1) / kCeThreads;  // 16-byte chunks per thread
+    if (per_thread <= 8)
+      ce_fwd_regs<T, 8><<<grid, block, 0, st>>>((int)V, (const T*)logits, map, labels, (T*)loss, lse);
+    else if (per_thread <= 16)
+      ce_fwd_regs<T, 16><<<grid, block, 0, st>>>((int)V, (const T*)logits, map, labels, (T*)loss, lse);
+    else if (per_thread <= 25)
+      ce_fwd_regs<T, 25><<<grid, block, 0, st>>>((int)V, (const T*)logits, map, labels, (T*)loss, lse);
+    else
+      ce_fwd<T, true><<<grid, block, 0, st>>>((int)V, (const T*)logits, map, labels, (T*)loss, lse);
+  } else
     ce_fwd<T, false><<<grid, block, 0, st>>>((int)V, (const T*)logits, map, labels, (T*)loss, lse);
   TF_CHECK_LAUNCH();
   return TF_OK;
