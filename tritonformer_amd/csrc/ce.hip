@@ -8,6 +8,12 @@ namespace tfa {
 
 constexpr int kCeThreads = 256;
 
+// v_exp_f32 as it is: the library exp2f wraps the same instruction in a range check and a rescaling
+// (five instructions more per element) that only matter for results below 2^-126, which are
+// flushed to zero here -- terms that change neither a sum of exponentials whose largest term is 1
+// nor a 16-bit gradient.
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
 struct MaxSum {
   float m;  // running max of x*log2e
   float s;  // running sum of exp2(x*log2e - m)
@@ -75,7 +81,7 @@ __global__ __launch_bounds__(kCeThreads) void ce_fwd(int V, const T* __restrict_
         if (cm > acc.m) { acc.s *= exp2f(acc.m - cm); acc.m = cm; }
         float part = 0.f;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) part += exp2f(v[e] * kLog2e - acc.m);
+        for (int e = 0; e < 8; ++e) part += fast_exp2(v[e] * kLog2e - acc.m);
         acc.s += part;
       }
     }
@@ -140,7 +146,7 @@ __global__ __launch_bounds__(kCeThreads) void ce_fwd_regs(int V, const T* __rest
       unpack8<T>(raw[u], v);
       float part = 0.f;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) part += exp2f(v[e] * kLog2e - m2);
+      for (int e = 0; e < 8; ++e) part += fast_exp2(v[e] * kLog2e - m2);
       s += part;
     }
   }
@@ -177,7 +183,7 @@ __global__ __launch_bounds__(kCeThreads) void ce_bwd(int V, const T* __restrict_
       float v[8];
       Chunk<T>::load(xr + c * 8, v);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) v[e] = exp2f(v[e] * kLog2e - l2);
+      for (int e = 0; e < 8; ++e) v[e] = fast_exp2(v[e] * kLog2e - l2);
       if ((lab >> 3) == c) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] -= (e == (lab & 7)) ? 1.0f : 0.0f;
