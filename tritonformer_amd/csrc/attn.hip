@@ -163,6 +163,37 @@ struct BiasTile {
 
 // (Register r of a 32x32 MFMA result covers row (r/4)*8 + 4*(lane/32) + r%4.)
 
+// Write-out of a wave's 32 x HD result held as 32x32 MFMA accumulators (register g*4+e of slice d,
+// lane l = row l%32, column d*32 + g*8 + 4*(l/32) + e): scaled, rounded, parked in a wave-private
+// LDS slab and read back row-contiguously, so that every global store instruction covers whole
+// 128-byte lines of complete rows (8 bytes per lane straight from the accumulators would fill each
+// line piecewise over eight instructions).  LDS accesses of one wave execute in order: no barrier.
+template <typename T, int HD>
+__device__ __forceinline__ void store_rows32(char* slab, T* dst, int64_t row_stride, const f32x16 (&acc)[HD / 32],
+                                             float scale, int lane) {
+  typedef typename Vec<T>::v4 v4;
+  constexpr int ROWB = HD * 2 + 16;  // padded row pitch in bytes
+  constexpr int CH = HD * 2 / 16;    // 16-byte chunks per row
+  constexpr int RPI = 64 / CH;       // rows covered by one wave-wide access
+#pragma unroll
+  for (int d = 0; d < HD / 32; ++d)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      v4 o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = (T)(acc[d][g * 4 + e] * scale);
+      *reinterpret_cast<v4*>(slab + (lane & 31) * ROWB + (d * 32 + g * 8 + 4 * (lane >> 5)) * 2) = o;
+    }
+#pragma unroll
+  for (int rr = 0; rr < 32 / RPI; ++rr) {
+    const int r = rr * RPI + lane / CH, c = lane % CH;
+    const u32x4 v = lds_ld16(slab, r * ROWB + c * 16);
+    if constexpr (HD >= 64) st16(dst + (int64_t)r * row_stride + c * 8, v);  // whole lines: written through
+    else *reinterpret_cast<u32x4*>(dst + (int64_t)r * row_stride + c * 8) = v;
+  }
+}
+
+
 // ===========================================================================
 // Forward.  Workgroup: 4 waves x 32 queries; key/value blocks of 64.
 //
@@ -189,6 +220,7 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (BMODE == kDenseBias ? 2 : 3)) v
   typedef typename Vec<T>::v4 v4;
   constexpr int KS = HD / 16, DT = HD / 32;
   constexpr int STAGE = 2 * KT::BYTES + (HAS_BIAS ? BiasTile::BYTES : 0);
+  static_assert(4 * 32 * (HD * 2 + 16) <= 2 * STAGE, "the result slabs of the four waves reuse the pipeline stages");
   constexpr int PT = KT::PER_THREAD;  // 16-byte chunks per thread per 64-row tile
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
@@ -381,15 +413,8 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (BMODE == kDenseBias ? 2 : 3)) v
     const float l_tot = lacc[0];
     const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
     if (lane < 32) p.lse[(int64_t)bh * p.S + myq] = m_ref + log2f(l_tot);
-#pragma unroll
-    for (int d = 0; d < DT; ++d)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        v4 o;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) o[e] = (T)(oacc[d][g * 4 + e] * inv);
-        *reinterpret_cast<v4*>(O + (int64_t)myq * p.oss + d * 32 + g * 8 + 4 * (lane >> 5)) = o;
-      }
+    // the pipeline stages are free: every wave is past the last barrier of the loop
+    store_rows32<T, HD>(smem + wave * (32 * (HD * 2 + 16)), O + (int64_t)q0w * p.oss, p.oss, oacc, inv, lane);
   }
 }
 
@@ -409,6 +434,7 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_dkdv_kernel(AttnPa
   constexpr int STAT = 2 * QT::BYTES, BIAS = STAT + 2 * 64 * 4;
   constexpr int BIAS_BYTES = 64 * 128 * 2;
   constexpr int STAGE = BIAS + (HAS_BIAS ? BIAS_BYTES : 0);
+  static_assert(4 * 32 * (HD * 2 + 16) <= 2 * STAGE, "the result slabs of the four waves reuse the pipeline stages");
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -609,20 +635,11 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_dkdv_kernel(AttnPa
   if (active) {
     T* dK = (T*)p.dk + base;
     T* dV = (T*)p.dv + base;
-#pragma unroll
-    for (int d = 0; d < DT; ++d)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        v4 a, c;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          a[e] = (T)(dk[d][g * 4 + e] * p.scale);
-          c[e] = (T)dv[d][g * 4 + e];
-        }
-        const int64_t off = (int64_t)mykey * p.ss + d * 32 + g * 8 + 4 * (lane >> 5);
-        *reinterpret_cast<v4*>(dK + off) = a;
-        *reinterpret_cast<v4*>(dV + off) = c;
-      }
+    // the pipeline stages are free: every wave is past the last barrier of the loop
+    char* slab = smem + wave * (32 * (HD * 2 + 16));
+    const int64_t row0 = (int64_t)(mykey - (lane & 31)) * p.ss;
+    store_rows32<T, HD>(slab, dK + row0, p.ss, dk, p.scale, lane);
+    store_rows32<T, HD>(slab, dV + row0, p.ss, dv, 1.0f, lane);
   }
 }
 
@@ -638,6 +655,7 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (BMODE != kNoBias ? 2 : 3)) void
   typedef typename Vec<T>::v4 v4;
   constexpr int KS = HD / 16, DT = HD / 32;
   constexpr int STAGE = 2 * KT::BYTES + (HAS_BIAS ? BiasTile::BYTES : 0);
+  static_assert(4 * 32 * (HD * 2 + 16) <= 2 * STAGE, "the result slabs of the four waves reuse the pipeline stages");
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -819,15 +837,9 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (BMODE != kNoBias ? 2 : 3)) void
 
   if (active) {
     T* dQ = (T*)p.dq + base;
-#pragma unroll
-    for (int d = 0; d < DT; ++d)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        v4 a;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) a[e] = (T)(dq[d][g * 4 + e] * p.scale);
-        *reinterpret_cast<v4*>(dQ + (int64_t)myq * p.ss + d * 32 + g * 8 + 4 * (lane >> 5)) = a;
-      }
+    // the pipeline stages are free: every wave is past the last barrier of the loop
+    store_rows32<T, HD>(smem + wave * (32 * (HD * 2 + 16)), dQ + (int64_t)(myq - (lane & 31)) * p.ss, p.ss, dq, p.scale,
+                        lane);
   }
 }
 

@@ -47,7 +47,27 @@ __device__ __forceinline__ float wave_max(float v) {
 
 // ---- 16-byte global access -------------------------------------------------
 __device__ __forceinline__ u32x4 ld16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
-__device__ __forceinline__ void st16(void* p, u32x4 v) { *reinterpret_cast<u32x4*>(p) = v; }
+// Result stores that cover whole cache lines (a wave writes complete 128-byte row segments) are
+// written through L2 at once (device scope) instead of staying dirty in the cache: a kernel then
+// ends with less left to write back, and the write traffic runs beside its remaining work
+// instead of in a burst after it (0.3-0.7 ms of a 27 ms training step of the 410M model).  Stores
+// that fill a line piecewise over several instructions must NOT use these: written through, every
+// piece becomes a partial-line write (the same step 2 ms slower with the attention results stored
+// this way).  The compiler does not see a store inside an asm statement, so the wait states that
+// a store needs before a VALU instruction may overwrite its data registers are part of the
+// statement.
+__device__ __forceinline__ void st16(void* p, u32x4 v) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ void st8(void* p, u32x2 v) {
+  asm volatile("global_store_dwordx2 %0, %1, off sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
+}
+// any 8- or 16-byte vector value
+template <typename V> __device__ __forceinline__ void store_out(void* p, const V& v) {
+  static_assert(sizeof(V) == 8 || sizeof(V) == 16, "8- or 16-byte values");
+  if constexpr (sizeof(V) == 16) st16(p, __builtin_bit_cast(u32x4, v));
+  else st8(p, __builtin_bit_cast(u32x2, v));
+}
 
 template <typename T> __device__ __forceinline__ void unpack8(u32x4 raw, float (&out)[8]) {
   typename Vec<T>::v8 h = __builtin_bit_cast(typename Vec<T>::v8, raw);

@@ -46,9 +46,10 @@ __global__ __launch_bounds__(256) void embed_fwd(int64_t T, int S, int d, int64_
       if constexpr (sizeof(TO) == 2) {
         Chunk<TO>::store(orow + c, a);
       } else {
-        float lo[4] = {a[0], a[1], a[2], a[3]}, hi[4] = {a[4], a[5], a[6], a[7]};
-        Chunk<float>::store((float*)orow + c, lo);
-        Chunk<float>::store((float*)orow + c + 4, hi);
+        // two 16-byte halves per lane: half lines per instruction, so plain (write-back) stores
+        const f32x4 lo = {a[0], a[1], a[2], a[3]}, hi = {a[4], a[5], a[6], a[7]};
+        *reinterpret_cast<f32x4*>((float*)orow + c) = lo;
+        *reinterpret_cast<f32x4*>((float*)orow + c + 4) = hi;
       }
     }
   } else {
@@ -154,9 +155,10 @@ __global__ __launch_bounds__(256) void embed_bwd(int T, int S, int d, int P, int
       if constexpr (sizeof(TP) == 2) {
         Chunk<TP>::store(dst + c, acc);
       } else {
-        float lo[4] = {acc[0], acc[1], acc[2], acc[3]}, hi[4] = {acc[4], acc[5], acc[6], acc[7]};
-        Chunk<float>::store((float*)dst + c, lo);
-        Chunk<float>::store((float*)dst + c + 4, hi);
+        // two 16-byte halves per lane: half lines per instruction, so plain (write-back) stores
+        const f32x4 lo = {acc[0], acc[1], acc[2], acc[3]}, hi = {acc[4], acc[5], acc[6], acc[7]};
+        *reinterpret_cast<f32x4*>((float*)dst + c) = lo;
+        *reinterpret_cast<f32x4*>((float*)dst + c + 4) = hi;
       }
     } else {
       dst[c] = (TP)acc[0];

@@ -659,7 +659,7 @@ __global__ __launch_bounds__(256) void gemm_reduce(int M, int N, int splits, con
       Quad qd;
 #pragma unroll
       for (int e = 0; e < 4; ++e) qd.v[e] = o[e];
-      *reinterpret_cast<Quad*>(C + (int64_t)m * ldc + n + (int64_t)(n / chunk_n) * chunk_skip) = qd;
+      store_out(C + (int64_t)m * ldc + n + (int64_t)(n / chunk_n) * chunk_skip, qd);
     }
   } else {
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
@@ -698,7 +698,7 @@ __global__ __launch_bounds__(256) void gemm_reduce_group(ReduceBatch batch) {
       Quad qd;
 #pragma unroll
       for (int e = 0; e < 4; ++e) qd.v[e] = (TO)s[e];
-      *reinterpret_cast<Quad*>(C + (int64_t)m * r.ldc + n + (int64_t)(n / r.chunk_n) * r.chunk_skip) = qd;
+      store_out(C + (int64_t)m * r.ldc + n + (int64_t)(n / r.chunk_n) * r.chunk_skip, qd);
     }
   } else {
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {

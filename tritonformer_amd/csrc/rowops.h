@@ -21,7 +21,7 @@ template <> struct Chunk<float> {
     f32x4 r;
 #pragma unroll
     for (int i = 0; i < 4; ++i) r[i] = v[i];
-    *reinterpret_cast<f32x4*>(p) = r;
+    store_out(p, r);
   }
 };
 
