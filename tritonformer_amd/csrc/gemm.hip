@@ -600,10 +600,20 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams& p, const int pid
   }
 
   if (p.flags & 8) return;
+  static_assert(NW * 32 * (WTN * 4 + 16) <= 2 * STAGE, "epilogue staging must fit in the pipeline LDS");
   if (p.splits > 1) {
-    gemm_epilogue<T, TM, TN, WTM, WTN, true>(p, acc, m0, n0, wm, wn, lane, split);
+    // fp32 partial of this contraction slice: a plain (M, N) matrix, written like an fp32 result
+    GemmParams q = p;
+    q.C = p.partial + (int64_t)split * p.M * p.N;
+    q.ldc = p.N;
+    q.bias = nullptr;
+    q.relu = 0;
+    q.mask = nullptr;
+    q.chunk_n = p.N;
+    q.chunk_skip = 0;
+    __syncthreads();  // all waves are done reading the last pipeline stage
+    gemm_epilogue_lds<T, float, TM, TN, WTM, WTN>(q, acc, smem, m0, n0, wm, wn, wave, lane);
   } else {
-    static_assert(NW * 32 * (WTN * 4 + 16) <= 2 * STAGE, "epilogue staging must fit in the pipeline LDS");
     __syncthreads();  // all waves are done reading the last pipeline stage
     if (p.out_f32) gemm_epilogue_lds<T, float, TM, TN, WTM, WTN>(p, acc, smem, m0, n0, wm, wn, wave, lane);
     else gemm_epilogue_lds<T, T, TM, TN, WTM, WTN>(p, acc, smem, m0, n0, wm, wn, wave, lane);
