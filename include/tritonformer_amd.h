@@ -100,6 +100,22 @@ int tf_gemm_out_chunked(void* stream, int dtype, int out_dtype, int layout_a, in
                         void* C, int64_t ldc, int64_t chunk_n, int64_t chunk_stride,
                         const void* bias, int relu, const void* mask_act, int64_t ld_mask,
                         void* workspace, int64_t workspace_bytes);
+/* tf_gemm_out with the ReLU mask carried as one bit per element instead of the
+ * activation itself.  Exactly one of bits_out / bits_in is given; rows of ld_bits
+ * bytes (>= N / 8, N a multiple of 8), element (m, n) is bit n % 8 of byte n / 8.
+ *   bits_out: C = relu(A . B + bias) in the operand dtype, bits_out = (C > 0)
+ *             (the forward of LinearNoBiasReLU / LinearBiasReLU, tritonformer/linear.py:47-102);
+ *   bits_in:  C = bit ? A . B : 0, no bias (mask_grad of kernels/activation.py:27-44
+ *             fused into dH = dY . W2^T, reading a sixteenth of what the activation holds).
+ * Served by the write-out of the direct-to-LDS kernels only: returns TF_EINVAL when
+ * their preconditions (16-byte aligned operands, extents and leading dimensions
+ * multiples of 8, K a multiple of 64) do not hold; callers then use tf_gemm_out with
+ * the activation as mask_act.  Needs no workspace. */
+int tf_gemm_relu_bits(void* stream, int dtype, int out_dtype, int layout_a, int layout_b,
+                      int64_t M, int64_t N, int64_t K,
+                      const void* A, int64_t lda, const void* B, int64_t ldb,
+                      void* C, int64_t ldc, const void* bias,
+                      void* bits_out, const void* bits_in, int64_t ld_bits);
 int64_t tf_gemm_workspace_bytes(int layout_a, int layout_b, int64_t M, int64_t N, int64_t K);
 
 /* `count` (1..4) independent products of one dtype and one pair of operand layouts,

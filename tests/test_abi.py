@@ -70,6 +70,17 @@ def test_gemm_rejects_bad_arguments():
     assert lib.tf_gemm_out(None, 0, 1, 0, 1, 64, 64, 64, *out_tail) == -2                       # bf16 out of fp16 in
     assert lib.tf_gemm_out(None, 0, 0, 0, 1, 64, 64, 64, FAKE, 64, FAKE, 64, FAKE, 64, None, 1, FAKE, 64,
                            None, 0) == -1                                                        # mask with ReLU
+    # ReLU sign bits: exactly one of bits_out / bits_in, N a multiple of 8, rows of at least N / 8 bytes,
+    # and only where the direct-to-LDS kernel runs (K a multiple of 64 among other things)
+    rb = lambda n, k, out, inp, ld: lib.tf_gemm_relu_bits(None, 0, 0, 0, 1, 64, n, k, FAKE, k, FAKE, n, FAKE, n, None,
+                                                          out, inp, ld)
+    assert rb(64, 64, None, None, 8) == -1 and rb(64, 64, FAKE, FAKE, 8) == -1
+    assert rb(60, 64, FAKE, None, 8) == -1 and rb(64, 64, FAKE, None, 7) == -1
+    assert rb(64, 72, FAKE, None, 8) == -1 and rb(64, 72, None, FAKE, 8) == -1
+    assert lib.tf_gemm_relu_bits(None, 0, 2, 0, 1, 64, 64, 64, FAKE, 64, FAKE, 64, FAKE, 64, None, FAKE, None,
+                                 8) == -1                                                        # bits_out with fp32 C
+    assert lib.tf_gemm_relu_bits(None, 0, 0, 0, 1, 64, 64, 64, FAKE, 64, FAKE, 64, FAKE, 64, FAKE, None, FAKE,
+                                 8) == -1                                                        # bits_in with bias
     # column-block output: blocks must divide N, be multiples of 8 wide and not overlap
     def chunked(chunk_n, chunk_stride, ldc=32):
         return lib.tf_gemm_out_chunked(None, 0, 2, 1, 1, 64, 96, 64, FAKE, 64, FAKE, 96, FAKE, ldc, chunk_n,

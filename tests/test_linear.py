@@ -306,3 +306,48 @@ def test_grouped_weight_gradients_equal_separate_products(case, dev):
             assert rel_l2(outs[0], ref) < 1e-4
     with pytest.raises(ValueError):
         K.mm_dw_group(pairs * 5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dims", [(2, 128, 256, 1024), (1, 384, 128, 320)])
+@pytest.mark.parametrize("use_bias", [False, True])
+def test_relu_sign_bits_equal_the_activation_mask(dims, use_bias, dev):
+    """gemm_relu_bits returns relu(x W + b) bit-identical to the plain ReLU GEMM, and one bit per
+    element that says where it is positive (bit n % 8 of byte n / 8); the masked product taken
+    from those bits equals the one that reads the activation (kernels/activation.py:27-44)."""
+    import numpy as np
+    from tritonformer_amd import kernels as K
+
+    b, m, d, f = dims
+    g = torch.Generator().manual_seed(31)
+    x = torch.randn(b, m, d, generator=g).half().to(dev)
+    w1 = (torch.randn(d, f, generator=g) / d ** 0.5).half().to(dev)
+    w2 = (torch.randn(f, d, generator=g) / f ** 0.5).half().to(dev)
+    b1 = torch.randn(f, generator=g).half().to(dev) if use_bias else None
+    dy = torch.randn(b, m, d, generator=g).half().to(dev)
+    hidden, bits = K.gemm_relu_bits(x, w1, b1)
+    assert bits is not None and bits.shape == (b * m, f // 8) and bits.dtype == torch.uint8
+    assert torch.equal(hidden, K.gemm(x, w1, b1, True))
+    expect = np.packbits((hidden.reshape(-1, f) > 0).cpu().numpy(), axis=1, bitorder="little")
+    assert np.array_equal(bits.cpu().numpy(), expect)
+    assert torch.equal(K.mm_masked_bits(dy, w2.T, bits), K.mm(dy, w2.T, mask_act=hidden))
+
+
+@pytest.mark.gpu
+def test_relu_sign_bits_fall_back_when_the_kernel_cannot_take_the_problem(dev):
+    """A contraction length that the direct-to-LDS kernel does not take: no bits, same result;
+    the fused MLP then masks with the activation and still matches the two-function form."""
+    from tritonformer_amd import kernels as K
+
+    g = torch.Generator().manual_seed(32)
+    x = torch.randn(1, 64, 72, generator=g).half().to(dev)
+    w1 = (torch.randn(72, 96, generator=g) / 8).half().to(dev)
+    w2 = (torch.randn(96, 72, generator=g) / 8).half().to(dev)
+    hidden, bits = K.gemm_relu_bits(x, w1, None)
+    assert bits is None and torch.equal(hidden, K.gemm(x, w1, None, True))
+    a = [t.clone().requires_grad_(True) for t in (x, w1, w2)]
+    T.mlp_fused_relu.apply(a[0], a[1], None, a[2], None).sum().backward()
+    c = [t.clone().requires_grad_(True) for t in (x, w1, w2)]
+    T.linear_no_bias.apply(T.linear_fused_relu.apply(c[0], c[1]), c[2]).sum().backward()
+    for ta, tb in zip(a, c):
+        assert torch.equal(ta.grad, tb.grad)

@@ -26,6 +26,8 @@ SIGNATURES = {
                          _vp, _i64]),
     "tf_gemm_out_chunked": (_i, [_vp, _i, _i, _i, _i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _i64, _i64,
                                  _vp, _i, _vp, _i64, _vp, _i64]),
+    "tf_gemm_relu_bits": (_i, [_vp, _i, _i, _i, _i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp,
+                               _i64]),
     "tf_cast_pack": (_i, [_vp, _i, _i, _i, _i64, _i64, _vp, _i64, _vp, _i64]),
     "tf_embedding_fwd": (_i, [_vp, _i, _i, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _i64, _vp, _i64]),
     "tf_embedding_bwd_workspace_bytes": (_i64, [_i64]),

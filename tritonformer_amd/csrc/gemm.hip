@@ -44,6 +44,12 @@ struct GemmParams {
   int out_f32;  // C holds fp32 instead of T
   const void* mask;  // optional (M, N) activation of type T: C = mask > 0 ? C : 0
   int64_t ldmask;
+  // One bit per element, rows of ldsign bytes, bit n % 8 of byte n / 8 (direct-to-LDS kernels only):
+  // sign_out receives C > 0 (with the ReLU epilogue: the gradient mask of the activation, at a
+  // sixteenth of its size); sign_in zeroes C where its bit is clear.
+  void* sign_out;
+  const void* sign_in;
+  int64_t ldsign;
   // Output split into column blocks of chunk_n columns, each its own (M, chunk_n) matrix
   // with leading dimension ldc, chunk_skip + chunk_n elements after the previous one.
   // One matrix: chunk_n = N, chunk_skip = 0.
@@ -404,7 +410,8 @@ struct DmaPanel {
 // tile) instead of 32 scattered 16-byte pieces.
 template <typename T, typename TO, int TM, int TN, int WTM, int WTN>
 __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x16 (&acc)[TM][TN], char* smem, int m0,
-                                                  int n0, int wm, int wn, int wave, int lane) {
+                                                  int n0, int wm, int wn, int wave, int lane,
+                                                  const uint8_t (*sign_bytes)[4] = nullptr) {
   constexpr int ES = (int)sizeof(TO);
   constexpr int ROWB = WTN * ES + 16;     // padded row pitch in bytes
   constexpr int CH = WTN * ES / 16;       // 16-byte chunks per row
@@ -468,6 +475,33 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x16 (&
             val = __builtin_bit_cast(u32x4, cv);
           }
         }
+        if (p.sign_in) {  // the same mask from one bit per element
+          unsigned bits;
+          if constexpr (ES == 2) bits = sign_bytes[i][rr];  // requested before the main loop
+          else bits = ((const uint8_t*)p.sign_in)[(int64_t)m * p.ldsign + (n >> 3)] >> (n & 7);
+          if constexpr (ES == 2) {
+            typename Vec<T>::v8 cv = __builtin_bit_cast(typename Vec<T>::v8, val);
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              if (!((bits >> e) & 1u)) cv[e] = (T)0.f;
+            val = __builtin_bit_cast(u32x4, cv);
+          } else {
+            f32x4 cv = __builtin_bit_cast(f32x4, val);
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (!((bits >> e) & 1u)) cv[e] = 0.f;
+            val = __builtin_bit_cast(u32x4, cv);
+          }
+        }
+        if constexpr (ES == 2) {
+          if (p.sign_out) {  // a chunk is 8 elements: one byte
+            const typename Vec<T>::v8 cv = __builtin_bit_cast(typename Vec<T>::v8, val);
+            unsigned bits = 0;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) bits |= ((float)cv[e] > 0.f ? 1u : 0u) << e;
+            ((uint8_t*)p.sign_out)[(int64_t)m * p.ldsign + (n >> 3)] = (uint8_t)bits;
+          }
+        }
         st16(C + c_index(p, m, n), val);
       }
     }
@@ -521,6 +555,22 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams& p, const int pid
     for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  // Mask bits of a 16-bit result: this lane's bytes (one per 8-element chunk it will store, in the
+  // order of the write-out) are requested here, a whole main loop ahead of their use -- loaded in
+  // the write-out they would sit between every LDS read and the store that needs both.
+  static_assert(64 / (WTN * 2 / 16) * 4 == 32, "four wave-wide stores per 32-row block of a 16-bit result");
+  uint8_t sign_bytes[TM][4] = {};
+  if (p.sign_in && !p.out_f32) {
+    constexpr int CH16 = WTN * 2 / 16, RPI16 = 64 / CH16;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) {
+        const int m = m0 + wm * WTM + i * 32 + rr * RPI16 + lane / CH16, n = n0 + wn * WTN + (lane % CH16) * 8;
+        if (m < p.M && n < p.N) sign_bytes[i][rr] = ((const uint8_t*)p.sign_in)[(int64_t)m * p.ldsign + (n >> 3)];
+      }
+  }
 
   // Bare s_barrier everywhere in the pipeline: __syncthreads() adds a fence that would
   // drain every outstanding direct-to-LDS load.  The waits that matter are explicit.
@@ -609,6 +659,8 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams& p, const int pid
     q.bias = nullptr;
     q.relu = 0;
     q.mask = nullptr;
+    q.sign_out = nullptr;
+    q.sign_in = nullptr;
     q.chunk_n = p.N;
     q.chunk_skip = 0;
     __syncthreads();  // all waves are done reading the last pipeline stage
@@ -616,7 +668,7 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams& p, const int pid
   } else {
     __syncthreads();  // all waves are done reading the last pipeline stage
     if (p.out_f32) gemm_epilogue_lds<T, float, TM, TN, WTM, WTN>(p, acc, smem, m0, n0, wm, wn, wave, lane);
-    else gemm_epilogue_lds<T, T, TM, TN, WTM, WTN>(p, acc, smem, m0, n0, wm, wn, wave, lane);
+    else gemm_epilogue_lds<T, T, TM, TN, WTM, WTN>(p, acc, smem, m0, n0, wm, wn, wave, lane, sign_bytes);
   }
 }
 
@@ -1018,12 +1070,18 @@ extern "C" int tf_gemm_out(void* stream, int dtype, int out_dtype, int layout_a,
                              relu, mask_act, ld_mask, workspace, workspace_bytes);
 }
 
-extern "C" int tf_gemm_out_chunked(void* stream, int dtype, int out_dtype, int layout_a, int layout_b, int64_t M,
-                                   int64_t N, int64_t K, const void* A, int64_t lda, const void* B, int64_t ldb,
-                                   void* C, int64_t ldc, int64_t chunk_n, int64_t chunk_stride, const void* bias,
-                                   int relu, const void* mask_act, int64_t ld_mask, void* workspace,
-                                   int64_t workspace_bytes) {
+static int gemm_entry(void* stream, int dtype, int out_dtype, int layout_a, int layout_b, int64_t M, int64_t N,
+                      int64_t K, const void* A, int64_t lda, const void* B, int64_t ldb, void* C, int64_t ldc,
+                      int64_t chunk_n, int64_t chunk_stride, const void* bias, int relu, const void* mask_act,
+                      int64_t ld_mask, void* workspace, int64_t workspace_bytes, void* sign_out, const void* sign_in,
+                      int64_t ld_sign) {
   if (!A || !B || !C) return TF_EINVAL;
+  const bool signs = sign_out || sign_in;
+  if (signs) {
+    if ((sign_out && sign_in) || mask_act || N % 8 != 0 || ld_sign < N / 8 || (chunk_n != 0 && chunk_n < N)) return TF_EINVAL;
+    if (sign_out && (!relu || out_dtype != dtype)) return TF_EINVAL;
+    if (sign_in && (bias || relu)) return TF_EINVAL;
+  }
   if (chunk_n < 0 || chunk_stride < 0) return TF_EINVAL;
   if (mask_act && (bias || relu || ld_mask < N)) return TF_EINVAL;
   if (out_dtype != dtype && out_dtype != TF_F32) return TF_EDTYPE;
@@ -1044,7 +1102,7 @@ extern "C" int tf_gemm_out_chunked(void* stream, int dtype, int out_dtype, int l
   const bool vec = aligned16(A) && aligned16(B) && aligned16(C) && (!bias || aligned16(bias)) && a_contig % 8 == 0 &&
                    b_contig % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 && N % 8 == 0 && ldc % 8 == 0 &&
                    (!mask_act || (aligned16(mask_act) && ld_mask % 8 == 0));
-  if (chunk_n == N) {
+  if (chunk_n == N && !signs) {
     const int64_t tail = tail_columns(M, N, K, vec, mask_act == nullptr);
     if (tail > 0) {  // whole rounds first, then the narrow remainder as a split contraction
       const int64_t n1 = N - tail;
@@ -1060,7 +1118,9 @@ extern "C" int tf_gemm_out_chunked(void* stream, int dtype, int out_dtype, int l
                                  workspace_bytes);
     }
   }
-  const GemmPlan pl = make_plan(M, N, K, vec, mask_act == nullptr);
+  const GemmPlan pl = make_plan(M, N, K, vec, mask_act == nullptr && !signs);
+  // the sign bits exist in the write-out of the direct-to-LDS kernels only
+  if (signs && !(kCfgs[pl.cfg].dma && vec && K % pl.bk == 0 && pl.splits == 1)) return TF_EINVAL;
   const int64_t need = pl.splits > 1 ? (int64_t)pl.splits * M * N * (int64_t)sizeof(float) : 0;
   if (need > 0 && (!workspace || workspace_bytes < need)) return TF_EWORKSPACE;
   if (need > 0 && !aligned16(workspace)) return TF_EALIGN;
@@ -1077,11 +1137,32 @@ extern "C" int tf_gemm_out_chunked(void* stream, int dtype, int out_dtype, int l
   p.out_f32 = out_dtype == TF_F32 ? 1 : 0;
   p.mask = mask_act;
   p.ldmask = ld_mask;
+  p.sign_out = sign_out;
+  p.sign_in = sign_in;
+  p.ldsign = ld_sign;
   p.chunk_n = (int)chunk_n;
   p.chunk_skip = chunk_stride - chunk_n;
   hipStream_t st = (hipStream_t)stream;
   if (dtype == TF_F16) return gemm_dispatch<f16>(st, layout_a, layout_b, vec, pl, p);
   return gemm_dispatch<bf16>(st, layout_a, layout_b, vec, pl, p);
+}
+
+extern "C" int tf_gemm_out_chunked(void* stream, int dtype, int out_dtype, int layout_a, int layout_b, int64_t M,
+                                   int64_t N, int64_t K, const void* A, int64_t lda, const void* B, int64_t ldb,
+                                   void* C, int64_t ldc, int64_t chunk_n, int64_t chunk_stride, const void* bias,
+                                   int relu, const void* mask_act, int64_t ld_mask, void* workspace,
+                                   int64_t workspace_bytes) {
+  return gemm_entry(stream, dtype, out_dtype, layout_a, layout_b, M, N, K, A, lda, B, ldb, C, ldc, chunk_n,
+                    chunk_stride, bias, relu, mask_act, ld_mask, workspace, workspace_bytes, nullptr, nullptr, 0);
+}
+
+extern "C" int tf_gemm_relu_bits(void* stream, int dtype, int out_dtype, int layout_a, int layout_b, int64_t M,
+                                 int64_t N, int64_t K, const void* A, int64_t lda, const void* B, int64_t ldb,
+                                 void* C, int64_t ldc, const void* bias, void* bits_out, const void* bits_in,
+                                 int64_t ld_bits) {
+  if (!bits_out && !bits_in) return TF_EINVAL;
+  return gemm_entry(stream, dtype, out_dtype, layout_a, layout_b, M, N, K, A, lda, B, ldb, C, ldc, 0, 0, bias,
+                    bits_out ? 1 : 0, nullptr, 0, nullptr, 0, bits_out, bits_in, ld_bits);
 }
 
 // ---- grouped products -------------------------------------------------------
@@ -1187,6 +1268,7 @@ extern "C" int tf_gemm_group(void* stream, int dtype, int out_dtype, int layout_
     p.flags = g_flags;
     p.out_f32 = out_dtype == TF_F32 ? 1 : 0;
     p.mask = nullptr; p.ldmask = 0;
+    p.sign_out = nullptr; p.sign_in = nullptr; p.ldsign = 0;
     p.chunk_n = (int)cn;
     p.chunk_skip = (cn == q.N ? q.N : q.chunk_stride) - cn;
     if (i < count) {

@@ -65,6 +65,14 @@ def _check_linear(a, b, bias=None):
     require_cuda(a, b, bias)
 
 
+def _operand_b(b, n, k):
+    if b.stride(-1) == 1 and b.stride(0) >= n:
+        return b, KMINOR, b.stride(0)          # (in, out) row-major: contraction strided
+    if b.stride(0) == 1 and b.stride(1) >= k:
+        return b, KMAJOR, b.stride(1)          # a transposed view, as linear.py:23 passes
+    return b.contiguous(), KMINOR, n
+
+
 def gemm(a, b, bias=None, fuse_relu=False, mask_act=None):
     """``relu?(a @ b + bias)`` for a (B, S, in), b (in, out) — reference ``mm``
     (kernels/gemm.py:361-401) and ``gemm`` (kernels/gemm.py:572-616).
@@ -81,17 +89,50 @@ def gemm(a, b, bias=None, fuse_relu=False, mask_act=None):
             mask_act = mask_act.contiguous()
     a2, m, k = _rows2d(a)
     n = b.shape[1]
-    if b.stride(-1) == 1 and b.stride(0) >= n:
-        lb, ldb = KMINOR, b.stride(0)          # (in, out) row-major: contraction strided
-    elif b.stride(0) == 1 and b.stride(1) >= k:
-        lb, ldb = KMAJOR, b.stride(1)          # a transposed view, as linear.py:23 passes
-    else:
-        b = b.contiguous()
-        lb, ldb = KMINOR, n
+    b, lb, ldb = _operand_b(b, n, k)
     if bias is not None and not bias.is_contiguous():
         bias = bias.contiguous()
     out = torch.empty(a.shape[:-1] + (n,), dtype=a.dtype, device=a.device)
     _gemm(a.dtype, KMAJOR, lb, m, n, k, a2, k, b, ldb, out, n, bias, fuse_relu, mask_act)
+    return out
+
+
+def gemm_relu_bits(a, b, bias=None):
+    """``relu(a @ b + bias)`` and its sign bits: a uint8 tensor (rows, out / 8), bit n % 8 of byte
+    n / 8 of a row set where the result is positive -- the ReLU gradient mask at a sixteenth of
+    the activation's size (reference mask_grad reads the activation, kernels/activation.py:27-44).
+    The bits are None when the kernel that produces them cannot take the problem."""
+    _check_linear(a, b, bias)
+    a2, m, k = _rows2d(a)
+    n = b.shape[1]
+    b, lb, ldb = _operand_b(b, n, k)
+    if bias is not None and not bias.is_contiguous():
+        bias = bias.contiguous()
+    out = torch.empty(a.shape[:-1] + (n,), dtype=a.dtype, device=a.device)
+    if n % 8 == 0:
+        bits = torch.empty((m, n // 8), dtype=torch.uint8, device=a.device)
+        rc = load().tf_gemm_relu_bits(stream_ptr(), dtype_code(a.dtype), dtype_code(a.dtype), KMAJOR, lb, m, n, k,
+                                      a2.data_ptr(), k, b.data_ptr(), ldb, out.data_ptr(), n,
+                                      bias.data_ptr() if bias is not None else None, bits.data_ptr(), None, n // 8)
+        if rc == 0:
+            return out, bits
+    _gemm(a.dtype, KMAJOR, lb, m, n, k, a2, k, b, ldb, out, n, bias, True, None)
+    return out, None
+
+
+def mm_masked_bits(a, b, bits):
+    """``(a @ b) * mask`` with the mask given as the sign bits of gemm_relu_bits."""
+    _check_linear(a, b, None)
+    a2, m, k = _rows2d(a)
+    n = b.shape[1]
+    if bits.dtype != torch.uint8 or bits.shape != (m, n // 8) or n % 8 or not bits.is_contiguous():
+        raise ValueError("bits must be the contiguous (rows, out / 8) uint8 tensor of gemm_relu_bits")
+    require_cuda(bits)
+    b, lb, ldb = _operand_b(b, n, k)
+    out = torch.empty(a.shape[:-1] + (n,), dtype=a.dtype, device=a.device)
+    check(load().tf_gemm_relu_bits(stream_ptr(), dtype_code(a.dtype), dtype_code(a.dtype), KMAJOR, lb, m, n, k,
+                                   a2.data_ptr(), k, b.data_ptr(), ldb, out.data_ptr(), n, None, None,
+                                   bits.data_ptr(), n // 8))
     return out
 
 

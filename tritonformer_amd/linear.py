@@ -4,11 +4,14 @@ import torch
 from torch.autograd import Function
 
 from ._amp import amp_bwd, amp_fwd
-from .kernels import cast_pack, gemm, mask_grad, mm, mm_dw, mm_dw_group, unbroadcast_leading
+from .kernels import (cast_pack, gemm, gemm_relu_bits, mask_grad, mm, mm_dw, mm_dw_group, mm_masked_bits,
+                      unbroadcast_leading)
 
 
 # True: weight gradients that are available together are computed by one grouped launch
 GROUP_DW = True
+# True: the fused MLP keeps the ReLU gradient mask as one bit per element, written by the first GEMM
+RELU_BITS = True
 # True: fp32 master weights of one block are converted to 16 bits by one kernel launch, not one each
 PACK_CASTS = True
 
@@ -120,9 +123,13 @@ class MLPReLU(Function):
                 w1, w2 = both[0, : w1.numel()].view(w1.shape), both[0, w1.numel():].view(w2.shape)
             else:
                 w1, w2 = w1.to(input.dtype), w2.to(input.dtype)
-        hidden = gemm(input, w1, b1, True)
+        if RELU_BITS:
+            hidden, bits = gemm_relu_bits(input, w1, b1)
+        else:
+            hidden, bits = gemm(input, w1, b1, True), None
         out = gemm(hidden, w2, b2, False)
         ctx.save_for_backward(input, w1, w2, hidden)
+        ctx.relu_bits = bits
         ctx.has_bias = (b1 is not None, b2 is not None)
         return out
 
@@ -131,7 +138,10 @@ class MLPReLU(Function):
     def backward(ctx, grad_output):
         input, w1, w2, hidden = ctx.saved_tensors
         f32 = torch.float32
-        grad_hidden = mm(grad_output, w2.T, mask_act=hidden)      # (dY W2^T) * (hidden > 0)
+        if ctx.relu_bits is not None:
+            grad_hidden = mm_masked_bits(grad_output, w2.T, ctx.relu_bits)  # (dY W2^T) * (hidden > 0)
+        else:
+            grad_hidden = mm(grad_output, w2.T, mask_act=hidden)
         grad_b2 = unbroadcast_leading(grad_output) if ctx.has_bias[1] else None
         grad_input = mm(grad_hidden, w1.T) if ctx.needs_input_grad[0] else None
         if GROUP_DW and ctx.arg_dtypes[1] == ctx.arg_dtypes[3]:
