@@ -74,7 +74,7 @@ def run_steps(model, tokens, n, dtype):
 
 
 class GemmTimer:
-    """HIP events on the current (launch) stream around every tf_gemm / tf_gemm_group call."""
+    """HIP events on the current (launch) stream around every tf_gemm / tf_gemm_relu_bits / tf_gemm_group call."""
 
     def __init__(self):
         self.records = []
@@ -104,13 +104,27 @@ class GemmTimer:
             key = ("group",) + tuple((q.M, q.N, q.K) for q in problems)
             self.records.append((key, e0, e1))
 
+        self._orig_bits = kernels._gemm_bits
+
+        def timed_bits(dtype, lb, m, n, k, *rest):
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record()
+            rc = self._orig_bits(dtype, lb, m, n, k, *rest)
+            e1.record()
+            if rc == 0:  # a refused call launched nothing; the caller falls back to _gemm
+                self.records.append((("bits", lb, m, n, k), e0, e1))
+            return rc
+
         kernels._gemm = timed
         kernels._gemm_group = timed_group
+        kernels._gemm_bits = timed_bits
         return self
 
     def __exit__(self, *exc):
         self._kernels._gemm = self._orig
         self._kernels._gemm_group = self._orig_group
+        self._kernels._gemm_bits = self._orig_bits
         torch.cuda.synchronize()
         self.by_shape = {}
         for key, e0, e1 in self.records:
@@ -309,7 +323,7 @@ def main():
             "flop_per_launch": round(gflops / launches, 1),
             "avg_launch_us": round(total_ms / launches * 1e3, 2),
             "gemm_ms_per_step": round(total_ms / reps, 3),
-            "measured": f"HIP events on the launch stream around each tf_gemm / tf_gemm_group call, {reps} instrumented steps "
+            "measured": f"HIP events on the launch stream around each tf_gemm / tf_gemm_relu_bits / tf_gemm_group call, {reps} instrumented steps "
                         "run after the timed ones (split-contraction launches include their reduce kernel)",
         }
     if args.calibrate_copy:

@@ -97,6 +97,15 @@ def gemm(a, b, bias=None, fuse_relu=False, mask_act=None):
     return out
 
 
+def _gemm_bits(dtype, lb, m, n, k, a, b, ldb, c, bias, bits_out, bits_in):
+    """One tf_gemm_relu_bits call (A contraction-contiguous); returns the status code."""
+    return load().tf_gemm_relu_bits(stream_ptr(), dtype_code(dtype), dtype_code(dtype), KMAJOR, lb, m, n, k,
+                                    a.data_ptr(), k, b.data_ptr(), ldb, c.data_ptr(), n,
+                                    bias.data_ptr() if bias is not None else None,
+                                    bits_out.data_ptr() if bits_out is not None else None,
+                                    bits_in.data_ptr() if bits_in is not None else None, n // 8)
+
+
 def gemm_relu_bits(a, b, bias=None):
     """``relu(a @ b + bias)`` and its sign bits: a uint8 tensor (rows, out / 8), bit n % 8 of byte
     n / 8 of a row set where the result is positive -- the ReLU gradient mask at a sixteenth of
@@ -111,9 +120,7 @@ def gemm_relu_bits(a, b, bias=None):
     out = torch.empty(a.shape[:-1] + (n,), dtype=a.dtype, device=a.device)
     if n % 8 == 0:
         bits = torch.empty((m, n // 8), dtype=torch.uint8, device=a.device)
-        rc = load().tf_gemm_relu_bits(stream_ptr(), dtype_code(a.dtype), dtype_code(a.dtype), KMAJOR, lb, m, n, k,
-                                      a2.data_ptr(), k, b.data_ptr(), ldb, out.data_ptr(), n,
-                                      bias.data_ptr() if bias is not None else None, bits.data_ptr(), None, n // 8)
+        rc = _gemm_bits(a.dtype, lb, m, n, k, a2, b, ldb, out, bias, bits, None)
         if rc == 0:
             return out, bits
     _gemm(a.dtype, KMAJOR, lb, m, n, k, a2, k, b, ldb, out, n, bias, True, None)
@@ -130,9 +137,7 @@ def mm_masked_bits(a, b, bits):
     require_cuda(bits)
     b, lb, ldb = _operand_b(b, n, k)
     out = torch.empty(a.shape[:-1] + (n,), dtype=a.dtype, device=a.device)
-    check(load().tf_gemm_relu_bits(stream_ptr(), dtype_code(a.dtype), dtype_code(a.dtype), KMAJOR, lb, m, n, k,
-                                   a2.data_ptr(), k, b.data_ptr(), ldb, out.data_ptr(), n, None, None,
-                                   bits.data_ptr(), n // 8))
+    check(_gemm_bits(a.dtype, lb, m, n, k, a2, b, ldb, out, None, None, bits))
     return out
 
 
