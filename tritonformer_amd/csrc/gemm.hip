@@ -20,6 +20,7 @@
 // Workgroup ids are remapped so that each of the 8 XCDs (which receive ids
 // round-robin) works on a compact block of neighbouring tiles and shares the
 // A/B panels through its own L2.
+#include <cstdio>
 #include <cstdlib>
 #include "rowops.h"
 
@@ -847,8 +848,30 @@ static GemmPlan plan_for(int cfg, int64_t M, int64_t N, int64_t K, double* cost_
   return pl;
 }
 
+// Diagnostic: TF_GEMM_RULE="M,N,K,cfg[;M,N,K,cfg...]" forces a tile configuration for the given extents only
+// (timing one product of a whole training step under another configuration).
+struct ShapeRule { int64_t m, n, k; int cfg; };
+static int load_rules(ShapeRule* out, int cap) {
+  const char* s = getenv("TF_GEMM_RULE");
+  int n = 0;
+  while (s && *s && n < cap) {
+    long long a, b, c; int cfg, used = 0;
+    if (sscanf(s, "%lld,%lld,%lld,%d%n", &a, &b, &c, &cfg, &used) != 4) break;
+    out[n++] = {a, b, c, cfg};
+    s += used;
+    if (*s == ';') ++s;
+  }
+  return n;
+}
+static ShapeRule g_rules[8];
+static const int g_num_rules = load_rules(g_rules, 8);
+
 static GemmPlan make_plan(int64_t M, int64_t N, int64_t K, bool vec, bool allow_split = true) {
   const bool dma = vec && K % 64 == 0;
+  for (int i = 0; i < g_num_rules; ++i)
+    if (g_rules[i].m == M && g_rules[i].n == N && g_rules[i].k == K && g_rules[i].cfg >= 0 && g_rules[i].cfg < kNumCfgs &&
+        (!kCfgs[g_rules[i].cfg].dma || dma))
+      return plan_for(g_rules[i].cfg, M, N, K, nullptr, allow_split);
   if (g_force_cfg >= 0 && g_force_cfg < kNumCfgs) {
     int cfg = g_force_cfg;
     if (kCfgs[cfg].dma && !dma) cfg = kCfgs[cfg].bm * kCfgs[cfg].bn >= 256 * 256 ? 0 : 1;  // register-staged twin
