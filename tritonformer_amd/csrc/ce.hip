@@ -68,7 +68,7 @@ __global__ __launch_bounds__(kCeThreads) void ce_fwd(int V, const T* __restrict_
       u32x4 raw[U];
 #pragma unroll
       for (int u = 0; u < U; ++u)
-        if (c0 + u * kCeThreads < nchunk) raw[u] = ld16(xr + (c0 + u * kCeThreads) * 8);
+        if (c0 + u * kCeThreads < nchunk) raw[u] = ld16_stream(xr + (c0 + u * kCeThreads) * 8);
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         if (c0 + u * kCeThreads >= nchunk) break;
@@ -117,7 +117,7 @@ __global__ __launch_bounds__(kCeThreads) void ce_fwd_regs(int V, const T* __rest
 #pragma unroll
   for (int u = 0; u < NCH; ++u) {
     const int c = threadIdx.x + u * kCeThreads;
-    if (c < nchunk) raw[u] = ld16(xr + c * 8);
+    if (c < nchunk) raw[u] = ld16_stream(xr + c * 8);
   }
   float m = -INFINITY;
 #pragma unroll
@@ -181,7 +181,7 @@ __global__ __launch_bounds__(kCeThreads) void ce_bwd(int V, const T* __restrict_
     const int nchunk = V >> 3;
     for (int c = threadIdx.x; c < nchunk; c += kCeThreads) {
       float v[8];
-      Chunk<T>::load(xr + c * 8, v);
+      Chunk<T>::load_stream(xr + c * 8, v);
 #pragma unroll
       for (int e = 0; e < 8; ++e) v[e] = fast_exp2(v[e] * kLog2e - l2);
       if ((lab >> 3) == c) {

@@ -47,6 +47,13 @@ __device__ __forceinline__ float wave_max(float v) {
 
 // ---- 16-byte global access -------------------------------------------------
 __device__ __forceinline__ u32x4 ld16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
+// Large data that a kernel reads exactly once (the logits of the cross-entropy passes, 0.8 GB): a
+// streaming (non-temporal) load, which leaves the caches to what is used again -- forward 195 ->
+// 150 us, backward 305 -> 273 us inside the training step.  No difference for the 34-67 MB inputs
+// of the normalisation, conversion and reduce passes, which keep plain loads.
+__device__ __forceinline__ u32x4 ld16_stream(const void* p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+}
 // Result stores that cover whole cache lines (a wave writes complete 128-byte row segments) are
 // written through L2 at once (device scope) instead of staying dirty in the cache: a kernel then
 // ends with less left to write back, and the write traffic runs beside its remaining work

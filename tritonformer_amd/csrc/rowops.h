@@ -8,6 +8,7 @@ namespace tfa {
 template <typename T> struct Chunk {  // 16-bit types: 8 elements per 16 bytes
   static constexpr int N = 8;
   static __device__ __forceinline__ void load(const T* p, float (&v)[8]) { unpack8<T>(ld16(p), v); }
+  static __device__ __forceinline__ void load_stream(const T* p, float (&v)[8]) { unpack8<T>(ld16_stream(p), v); }
   static __device__ __forceinline__ void store(T* p, const float (&v)[8]) { st16(p, pack8<T>(v)); }
 };
 template <> struct Chunk<float> {
