@@ -351,3 +351,24 @@ def test_relu_sign_bits_fall_back_when_the_kernel_cannot_take_the_problem(dev):
     T.linear_no_bias.apply(T.linear_fused_relu.apply(c[0], c[1]), c[2]).sum().backward()
     for ta, tb in zip(a, c):
         assert torch.equal(ta.grad, tb.grad)
+
+
+@pytest.mark.gpu
+def test_product_cut_into_whole_rounds_and_remainder(dev):
+    """8192 x 3072 x 1024 (the packed q/k/v projection of the 410M model) runs as one round of
+    256 x 256 tiles over the first 2048 columns plus the last 1024 columns as a product of their
+    own.  Every output element is the same contraction either way: the result must equal, bit for
+    bit, the two column blocks computed by separate calls, bias and ReLU included, and match the
+    fp32 oracle."""
+    from tritonformer_amd import kernels as K
+
+    g = torch.Generator().manual_seed(41)
+    x = torch.randn(4, 2048, 1024, generator=g).half().to(dev)
+    w = (torch.randn(1024, 3072, generator=g) * 0.02).half().to(dev)
+    bias = torch.randn(3072, generator=g).half().to(dev)
+    for b_, relu in ((None, False), (bias, True)):
+        y = K.gemm(x, w, b_, relu)
+        left = K.gemm(x, w[:, :2048].contiguous(), None if b_ is None else b_[:2048].contiguous(), relu)
+        right = K.gemm(x, w[:, 2048:].contiguous(), None if b_ is None else b_[2048:].contiguous(), relu)
+        assert torch.equal(y[..., :2048], left) and torch.equal(y[..., 2048:], right)
+        assert_close(y, R.linear(x, w, b_, relu), name="y")

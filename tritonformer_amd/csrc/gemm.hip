@@ -866,8 +866,10 @@ static int load_rules(ShapeRule* out, int cap) {
 static ShapeRule g_rules[8];
 static const int g_num_rules = load_rules(g_rules, 8);
 
-static GemmPlan make_plan(int64_t M, int64_t N, int64_t K, bool vec, bool allow_split = true) {
+static GemmPlan make_plan(int64_t M, int64_t N, int64_t K, bool vec, bool allow_split = true,
+                          double* cost_us = nullptr) {
   const bool dma = vec && K % 64 == 0;
+  if (cost_us) *cost_us = -1.0;  // stays negative when the configuration is forced
   for (int i = 0; i < g_num_rules; ++i)
     if (g_rules[i].m == M && g_rules[i].n == N && g_rules[i].k == K && g_rules[i].cfg >= 0 && g_rules[i].cfg < kNumCfgs &&
         (!kCfgs[g_rules[i].cfg].dma || dma))
@@ -890,6 +892,7 @@ static GemmPlan make_plan(int64_t M, int64_t N, int64_t K, bool vec, bool allow_
     const GemmPlan pl = plan_for(cand[i], M, N, K, &c, allow_split);
     if (c < best_cost) { best_cost = c; best = pl; }
   }
+  if (cost_us) *cost_us = best_cost;
   return best;
 }
 
@@ -1041,17 +1044,43 @@ extern "C" int tf_gemm_debug_flags(int flags) {
 // of tail columns, 0 for no cut.
 static int64_t tail_columns(int64_t M, int64_t N, int64_t K, bool vec, bool allow_split) {
   if (!allow_split || g_force_cfg >= 0 || g_force_splits > 0 || K < 32 * 64 || (g_flags & 64)) return 0;
-  const GemmPlan pl = make_plan(M, N, K, vec, allow_split);
-  if (pl.cfg != 2 || pl.splits != 1) return 0;
-  const int64_t tiles = (int64_t)pl.tiles_m * pl.tiles_n;
-  const int64_t rem = tiles % 256;
-  if (tiles <= 256 || rem == 0 || rem > 64) return 0;
-  int64_t a = pl.tiles_m, b = 256;
+  double uncut;
+  const GemmPlan pl = make_plan(M, N, K, vec, allow_split, &uncut);
+  const int64_t tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
+  int64_t a = tiles_m, b = 256;
   while (b) { const int64_t t = a % b; a = b; b = t; }
   const int64_t unit = 256 / a;  // tile columns per whole number of rounds
-  const int64_t tn1 = (pl.tiles_n / unit) * unit;
-  if (tn1 <= 0 || tn1 >= pl.tiles_n) return 0;
-  return N - tn1 * 256;
+  const int64_t tn1 = (tiles_n / unit) * unit;
+  if (tn1 <= 0 || tn1 * 256 >= N) return 0;
+  if (pl.cfg == 2 && pl.splits == 1) {
+    const int64_t tiles = tiles_m * tiles_n;
+    const int64_t rem = tiles % 256;
+    if (tiles > 256 && rem != 0 && rem <= 64) return N - tn1 * 256;
+  }
+  return 0;
+}
+
+// The same cut for a short contraction, by the cost model: whole rounds of 256x256 tiles, then
+// the remaining columns as a product of their own with whatever tiling suits them, when the two
+// together are cheaper than the best single launch (q/k/v projection 8192 x 3072 x 1024: one
+// round of 256x256 tiles + 1024 columns of 128x128 tiles, 0.2 ms per training step less than
+// three rounds of 128x128 tiles).
+static int64_t round_cut_columns(int64_t M, int64_t N, int64_t K, bool vec, bool allow_split) {
+  if (!allow_split || g_force_cfg >= 0 || g_force_splits > 0 || !(vec && K % 64 == 0) || (g_flags & 64)) return 0;
+  double uncut, whole, rest;
+  (void)make_plan(M, N, K, vec, allow_split, &uncut);
+  if (uncut < 0) return 0;
+  const int64_t tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
+  if (tiles_m * tiles_n <= 256) return 0;
+  int64_t a = tiles_m, b = 256;
+  while (b) { const int64_t t = a % b; a = b; b = t; }
+  const int64_t unit = 256 / a;
+  const int64_t tn1 = (tiles_n / unit) * unit;
+  if (tn1 <= 0 || tn1 * 256 >= N) return 0;
+  (void)plan_for(2, M, tn1 * 256, K, &whole, false);
+  (void)make_plan(M, N - tn1 * 256, K, vec, allow_split, &rest);
+  if (rest < 0) return 0;
+  return whole + rest + 3.0 < uncut ? N - tn1 * 256 : 0;
 }
 
 static int64_t single_need(int64_t M, int64_t N, int64_t K, bool vec) {
@@ -1067,7 +1096,8 @@ extern "C" int64_t tf_gemm_workspace_bytes(int layout_a, int layout_b, int64_t M
   int64_t need = 0;
   for (int vec = 0; vec < 2; ++vec) {
     int64_t n = single_need(M, N, K, vec != 0);
-    const int64_t tail = tail_columns(M, N, K, vec != 0, true);
+    int64_t tail = tail_columns(M, N, K, vec != 0, true);
+    if (tail == 0) tail = round_cut_columns(M, N, K, vec != 0, true);
     if (tail > 0) {
       const int64_t n1 = single_need(M, N - tail, K, vec != 0), n2 = single_need(M, tail, K, vec != 0);
       if (n1 > n) n = n1;
@@ -1126,7 +1156,8 @@ static int gemm_entry(void* stream, int dtype, int out_dtype, int layout_a, int 
                    b_contig % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 && N % 8 == 0 && ldc % 8 == 0 &&
                    (!mask_act || (aligned16(mask_act) && ld_mask % 8 == 0));
   if (chunk_n == N && !signs) {
-    const int64_t tail = tail_columns(M, N, K, vec, mask_act == nullptr);
+    int64_t tail = tail_columns(M, N, K, vec, mask_act == nullptr);
+    if (tail == 0) tail = round_cut_columns(M, N, K, vec, mask_act == nullptr);
     if (tail > 0) {  // whole rounds first, then the narrow remainder as a split contraction
       const int64_t n1 = N - tail;
       const int64_t osz = out_dtype == TF_F32 ? 4 : 2;
