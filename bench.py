@@ -29,7 +29,7 @@ PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per GEMM launch at the headline workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # scaled against a streaming kernel of known size (profiles/gemm_hbm_traffic_410m_step.md)
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = {"gpt2-410m-ctx2048-bs4": 164.4e6}
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = {"gpt2-410m-ctx2048-bs4": 149.2e6}
 
 WORKLOADS = {
     # name: (layers, d, heads, head_dim, ffn, seq, batch, linear_bias, alibi)
@@ -305,9 +305,13 @@ def main():
 
     if not args.no_roofline:
         reps = max(1, min(args.steps, 5))
+        from tritonformer_amd import _lib
+
+        count0 = _lib.load().tf_gemm_launch_count()
         with GemmTimer() as gt:
             run_steps(model, tokens, reps, dtype)
-        launches = sum(c for c, _ in gt.by_shape.values())
+        calls = sum(c for c, _ in gt.by_shape.values())
+        launches = _lib.load().tf_gemm_launch_count() - count0  # kernels: a product cut along N is two
         total_ms = sum(t for _, t in gt.by_shape.values())
         gflops = gemm_flops(L, d, f, S, B) * reps
         achieved = gflops / (total_ms * 1e-3) / 1e12
@@ -320,11 +324,13 @@ def main():
             "frac": round(achieved / PEAK_FP16_TFLOPS, 4),
             "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload),
             "launches_per_step": launches // reps,
+            "calls_per_step": calls // reps,
             "flop_per_launch": round(gflops / launches, 1),
             "avg_launch_us": round(total_ms / launches * 1e3, 2),
             "gemm_ms_per_step": round(total_ms / reps, 3),
             "measured": f"HIP events on the launch stream around each tf_gemm / tf_gemm_relu_bits / tf_gemm_group call, {reps} instrumented steps "
-                        "run after the timed ones (split-contraction launches include their reduce kernel)",
+                        "run after the timed ones; the event time of a call covers its GEMM kernel(s) and, for a split contraction, "
+                        "the reduce kernel; launches = GEMM kernels counted by the library",
         }
     if args.calibrate_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device=device).normal_()

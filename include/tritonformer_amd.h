@@ -137,6 +137,10 @@ int tf_gemm_group(void* stream, int dtype, int out_dtype, int layout_a, int layo
                   const tf_gemm_problem* problems, void* workspace, int64_t workspace_bytes);
 int64_t tf_gemm_group_workspace_bytes(int layout_a, int layout_b, int count,
                                       const tf_gemm_problem* problems);
+/* Diagnostic: number of GEMM kernels launched by this library since it was loaded (the reduce
+ * passes of split contractions are not counted; one tf_gemm* call may launch two kernels when
+ * the product is cut along N).  No counterpart in the reference. */
+int64_t tf_gemm_launch_count(void);
 /* Diagnostic, no counterpart in the reference (whose Triton autotuner picks
  * tiles per shape, kernels/gemm.py:15-79): force tile configuration `cfg`
  * (-1 = automatic) and contraction split `splits` (0 = automatic) for all

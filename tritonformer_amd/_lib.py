@@ -38,6 +38,7 @@ SIGNATURES = {
     "tf_gemm_group": (_i, [_vp, _i, _i, _i, _i, _i, _vp, _vp, _i64]),
     "tf_gemm_group_workspace_bytes": (_i64, [_i, _i, _i, _vp]),
     "tf_gemm_workspace_bytes": (_i64, [_i, _i, _i64, _i64, _i64]),
+    "tf_gemm_launch_count": (_i64, []),
     "tf_gemm_tune": (_i, [_i, _i]),
     "tf_gemm_debug_flags": (_i, [_i]),
     "tf_attn_fwd": (_i, [_vp, _i, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64,

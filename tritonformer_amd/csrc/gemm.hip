@@ -20,6 +20,7 @@
 // Workgroup ids are remapped so that each of the 8 XCDs (which receive ids
 // round-robin) works on a compact block of neighbouring tiles and shares the
 // A/B panels through its own L2.
+#include <atomic>
 #include <cstdio>
 #include <cstdlib>
 #include "rowops.h"
@@ -896,6 +897,9 @@ static GemmPlan make_plan(int64_t M, int64_t N, int64_t K, bool vec, bool allow_
   return best;
 }
 
+// Diagnostic: GEMM kernel launches since the library was loaded (reduce passes not counted).
+static std::atomic<int64_t> g_gemm_launches{0};
+
 template <typename K>
 static void allow_big_lds(K kernel, int bytes) {
   if (bytes > 64 * 1024)
@@ -913,6 +917,7 @@ static int launch_one(hipStream_t st, const GemmParams& p) {
   const unsigned grid = (unsigned)(p.tiles_m * p.tiles_n * p.splits);
   kernel<<<dim3(grid), dim3(WM * WN * 64), lds, st>>>(p);
   TF_CHECK_LAUNCH();
+  g_gemm_launches.fetch_add(1, std::memory_order_relaxed);
   return TF_OK;
 }
 
@@ -926,6 +931,7 @@ static int launch_dma(hipStream_t st, const GemmParams& p) {
   const unsigned grid = (unsigned)(p.tiles_m * p.tiles_n * p.splits);
   kernel<<<dim3(grid), dim3(WM * WN * 64), lds, st>>>(p);
   TF_CHECK_LAUNCH();
+  g_gemm_launches.fetch_add(1, std::memory_order_relaxed);
   return TF_OK;
 }
 
@@ -993,6 +999,7 @@ static int gemm_group_dispatch(hipStream_t st, const GemmGroup& g) {
   (void)once;
   kernel<<<dim3((unsigned)g.first[g.count]), dim3(512), lds, st>>>(g);
   TF_CHECK_LAUNCH();
+  g_gemm_launches.fetch_add(1, std::memory_order_relaxed);
   // second pass of the split contractions: all products of the group in one launch
   ReduceBatch rb = {};
   bool any = false, v4 = true;
@@ -1030,6 +1037,8 @@ extern "C" int tf_gemm_tune(int cfg, int splits) {
   g_force_splits = splits;
   return TF_OK;
 }
+
+extern "C" int64_t tf_gemm_launch_count(void) { return g_gemm_launches.load(std::memory_order_relaxed); }
 
 // Diagnostic: bit 0 skips the XCD remap, bit 3 skips the epilogue (timing only, wrong results).
 extern "C" int tf_gemm_debug_flags(int flags) {
