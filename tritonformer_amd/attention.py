@@ -143,6 +143,7 @@ class AttentionBlock(Function):
         grads = tuple(dqkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
         flash_wrapper_bwd(d_attn, attn.view(b, s, nh, hd).permute(0, 2, 1, 3), q, k, v, lse, attn_bias, grads=grads)
         dqkv = dqkv.view(b, s, 3 * nh * hd)
-        grad_x = mm(dqkv, w_qkv.T) if ctx.needs_input_grad[0] else None
+        # weight gradients first, the input gradient (what the next kernel reads) last
         d_wqkv, d_wo = mm_dw_group([(x, dqkv), (attn, grad_output)], out_dtype=ctx.weight_dtype, chunks=[3, 1])
+        grad_x = mm(dqkv, w_qkv.T) if ctx.needs_input_grad[0] else None
         return grad_x, d_wqkv[0], d_wqkv[1], d_wqkv[2], d_wo, None, None

@@ -20,13 +20,14 @@ def _grads(ctx, grad_output, inputs, weights):
     """dX = dY W^T (W read as stored, contraction along its rows) and
     dW = X^T dY with the batch folded into the contraction
     (reference linear.py:21-25 goes through bmm + torch.sum)."""
-    grad_input = mm(grad_output, weights.T) if ctx.needs_input_grad[0] else None
     grad_weights = None
     if ctx.needs_input_grad[1]:
         # an fp32 master weight (cast to 16 bit by autocast on the way in) gets its
         # gradient straight from the fp32 accumulators instead of a rounded copy
         master = torch.float32 if ctx.arg_dtypes[1] == torch.float32 else None
         grad_weights = mm_dw(inputs, grad_output, out_dtype=master)
+    # the input gradient last: it is what the next kernel of the backward pass reads
+    grad_input = mm(grad_output, weights.T) if ctx.needs_input_grad[0] else None
     return grad_input, grad_weights
 
 
@@ -143,7 +144,8 @@ class MLPReLU(Function):
         else:
             grad_hidden = mm(grad_output, w2.T, mask_act=hidden)
         grad_b2 = unbroadcast_leading(grad_output) if ctx.has_bias[1] else None
-        grad_input = mm(grad_hidden, w1.T) if ctx.needs_input_grad[0] else None
+        # the weight gradients first, the input gradient last: what the next kernel of the backward
+        # pass reads is then what was written last (0.1 ms per step of the 410M model)
         if GROUP_DW and ctx.arg_dtypes[1] == ctx.arg_dtypes[3]:
             # both weight gradients side by side in one launch
             grad_w1, grad_w2 = mm_dw_group([(input, grad_hidden), (hidden, grad_output)],
@@ -152,6 +154,7 @@ class MLPReLU(Function):
             grad_w2 = mm_dw(hidden, grad_output, out_dtype=f32 if ctx.arg_dtypes[3] == f32 else None)
             grad_w1 = mm_dw(input, grad_hidden, out_dtype=f32 if ctx.arg_dtypes[1] == f32 else None)
         grad_b1 = unbroadcast_leading(grad_hidden) if ctx.has_bias[0] else None
+        grad_input = mm(grad_hidden, w1.T) if ctx.needs_input_grad[0] else None
         return grad_input, grad_w1, grad_b1, grad_w2, grad_b2
 
 
@@ -177,6 +180,6 @@ class PackedLinearNoBias(Function):
     @amp_bwd
     def backward(ctx, grad_output):
         input, packed = ctx.saved_tensors
-        grad_input = mm(grad_output, packed.T) if ctx.needs_input_grad[0] else None
         grad_w = mm_dw(input, grad_output, out_dtype=ctx.weight_dtype, chunks=ctx.count)
+        grad_input = mm(grad_output, packed.T) if ctx.needs_input_grad[0] else None
         return (grad_input,) + tuple(grad_w[j] for j in range(ctx.count))
