@@ -423,6 +423,17 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x16 (&
   const T* bias = (const T*)p.bias;
   TO* C = (TO*)p.C;
   const int nbase = n0 + wn * WTN;
+  // this lane's bias values: the same for every 32-row block, requested once ahead of the loop
+  typename Vec<T>::v4 bvals[TN][4] = {};
+  if (bias) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int nl = j * 32 + g * 8 + (lane >> 5) * 4;
+        if (nbase + nl < p.N) bvals[j][g] = *reinterpret_cast<const typename Vec<T>::v4*>(bias + nbase + nl);
+      }
+  }
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -433,10 +444,9 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x16 (&
         float v[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[e] = acc[i][j][g * 4 + e];
-        if (bias && nbase + nl < p.N) {
-          const typename Vec<T>::v4 bv = *reinterpret_cast<const typename Vec<T>::v4*>(bias + nbase + nl);
+        if (bias) {
 #pragma unroll
-          for (int e = 0; e < 4; ++e) v[e] += (float)bv[e];
+          for (int e = 0; e < 4; ++e) v[e] += (float)bvals[j][g][e];
         }
         if (p.relu) {
 #pragma unroll
