@@ -410,7 +410,9 @@ struct DmaPanel {
 // reads it back row-contiguously, so every global store instruction writes whole
 // 16-byte chunks of complete row segments (8 rows x 128 B for a 64-wide wave
 // tile) instead of 32 scattered 16-byte pieces.
-template <typename T, typename TO, int TM, int TN, int WTM, int WTN>
+// PLAIN: the caller knows that there is no bias, ReLU, mask or sign-bit work (most launches of a
+// training step): the write-out is then straight-line code without the tests for them.
+template <typename T, typename TO, int TM, int TN, int WTM, int WTN, bool PLAIN = false>
 __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x16 (&acc)[TM][TN], char* smem, int m0,
                                                   int n0, int wm, int wn, int wave, int lane,
                                                   const uint8_t (*sign_bytes)[4] = nullptr) {
@@ -420,7 +422,11 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x16 (&
   constexpr int RPI = 64 / CH;            // rows covered by one wave-wide access
   constexpr int EPC = 16 / ES;            // elements per chunk
   char* mine = smem + wave * (32 * ROWB);
-  const T* bias = (const T*)p.bias;
+  const T* bias = PLAIN ? nullptr : (const T*)p.bias;
+  const bool relu = !PLAIN && p.relu;
+  const void* mask = PLAIN ? nullptr : p.mask;
+  const void* sign_in = PLAIN ? nullptr : p.sign_in;
+  void* sign_out = PLAIN ? nullptr : p.sign_out;
   TO* C = (TO*)p.C;
   const int nbase = n0 + wn * WTN;
   // this lane stores the same 16-byte column chunk of every row it handles: the column part of the
@@ -453,7 +459,7 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x16 (&
 #pragma unroll
           for (int e = 0; e < 4; ++e) v[e] += (float)bvals[j][g][e];
         }
-        if (p.relu) {
+        if (relu) {
 #pragma unroll
           for (int e = 0; e < 4; ++e) v[e] = fmaxf(v[e], 0.f);
         }
@@ -474,8 +480,8 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x16 (&
       u32x4 val = lds_ld16(mine, r * ROWB + c * 16);
       const int m = m0 + wm * WTM + i * 32 + r, n = nbase + c * EPC;
       if (m < p.M && n < p.N) {
-        if (p.mask) {  // ReLU gradient mask fused into the write-out: zero where the activation is not positive
-          const T* mk = (const T*)p.mask + (int64_t)m * p.ldmask + n;
+        if (mask) {  // ReLU gradient mask fused into the write-out: zero where the activation is not positive
+          const T* mk = (const T*)mask + (int64_t)m * p.ldmask + n;
           if constexpr (ES == 2) {
             const typename Vec<T>::v8 mv = __builtin_bit_cast(typename Vec<T>::v8, ld16(mk));
             typename Vec<T>::v8 cv = __builtin_bit_cast(typename Vec<T>::v8, val);
@@ -492,10 +498,10 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x16 (&
             val = __builtin_bit_cast(u32x4, cv);
           }
         }
-        if (p.sign_in) {  // the same mask from one bit per element
+        if (sign_in) {  // the same mask from one bit per element
           unsigned bits;
           if constexpr (ES == 2) bits = sign_bytes[i][rr];  // requested before the main loop
-          else bits = ((const uint8_t*)p.sign_in)[(int64_t)m * p.ldsign + (n >> 3)] >> (n & 7);
+          else bits = ((const uint8_t*)sign_in)[(int64_t)m * p.ldsign + (n >> 3)] >> (n & 7);
           if constexpr (ES == 2) {
             typename Vec<T>::v8 cv = __builtin_bit_cast(typename Vec<T>::v8, val);
 #pragma unroll
@@ -511,12 +517,12 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x16 (&
           }
         }
         if constexpr (ES == 2) {
-          if (p.sign_out) {  // a chunk is 8 elements: one byte
+          if (sign_out) {  // a chunk is 8 elements: one byte
             const typename Vec<T>::v8 cv = __builtin_bit_cast(typename Vec<T>::v8, val);
             unsigned bits = 0;
 #pragma unroll
             for (int e = 0; e < 8; ++e) bits |= ((float)cv[e] > 0.f ? 1u : 0u) << e;
-            ((uint8_t*)p.sign_out)[(int64_t)m * p.ldsign + (n >> 3)] = (uint8_t)bits;
+            ((uint8_t*)sign_out)[(int64_t)m * p.ldsign + (n >> 3)] = (uint8_t)bits;
           }
         }
         st16(C + (int64_t)m * p.ldc + col_off, val);
@@ -681,11 +687,17 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams& p, const int pid
     q.chunk_n = p.N;
     q.chunk_skip = 0;
     __syncthreads();  // all waves are done reading the last pipeline stage
-    gemm_epilogue_lds<T, float, TM, TN, WTM, WTN>(q, acc, smem, m0, n0, wm, wn, wave, lane);
+    gemm_epilogue_lds<T, float, TM, TN, WTM, WTN, true>(q, acc, smem, m0, n0, wm, wn, wave, lane);
   } else {
     __syncthreads();  // all waves are done reading the last pipeline stage
-    if (p.out_f32) gemm_epilogue_lds<T, float, TM, TN, WTM, WTN>(p, acc, smem, m0, n0, wm, wn, wave, lane);
-    else gemm_epilogue_lds<T, T, TM, TN, WTM, WTN>(p, acc, smem, m0, n0, wm, wn, wave, lane, sign_bytes);
+    const bool plain = !p.bias && !p.relu && !p.mask && !p.sign_in && !p.sign_out;
+    if (p.out_f32) {
+      if (plain) gemm_epilogue_lds<T, float, TM, TN, WTM, WTN, true>(p, acc, smem, m0, n0, wm, wn, wave, lane);
+      else gemm_epilogue_lds<T, float, TM, TN, WTM, WTN>(p, acc, smem, m0, n0, wm, wn, wave, lane);
+    } else {
+      if (plain) gemm_epilogue_lds<T, T, TM, TN, WTM, WTN, true>(p, acc, smem, m0, n0, wm, wn, wave, lane);
+      else gemm_epilogue_lds<T, T, TM, TN, WTM, WTN>(p, acc, smem, m0, n0, wm, wn, wave, lane, sign_bytes);
+    }
   }
 }
 
