@@ -6,8 +6,17 @@ weights, every Linear / LayerNorm / attention / cross-entropy running on the
 tritonformer_amd HIP kernels.  Prints one JSON line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
+                    [--no-extras] [--gemm-table FILE]
 
-value        = algorithmic FLOPs of the step (6*T*P_mat + 7*L*B*S^2*d) / step time, in TFLOP/s
+value        = algorithmic FLOPs of the step (6*T*P_mat + 7*L*B*S^2*d) / step time, in TFLOP/s, for the
+               reference's protocol (README.md:62-77: forward under autocast, `loss.backward()` unscaled,
+               no optimizer), the 16-bit copies of the unchanged fp32 master weights kept between steps
+               (the reference holds fp16 parameters and converts nothing)
+extras       = the same step timed in the other regimes, in the same run: `loss_scaled` (backward of
+               loss * 1024: without scaling, fp16 flushes most of the 1/N-scaled logit gradients to
+               zero and the backward GEMMs multiply near-constant operands, which the matrix cores run
+               at a higher clock), `recast_each_step` (weights converted in every forward pass), and
+               `workloads` (the other configurations of the baseline)
 roofline     = the GEMM kernel (dominant in time): algorithmic FLOPs per launch / mean launch
                duration, the duration measured with HIP events recorded on the launch stream
                around every GEMM launch in instrumented repeats of the same steps
@@ -63,14 +72,62 @@ def make_model(name, device, dtype):
     return model, tokens
 
 
-def run_steps(model, tokens, n, dtype):
+def run_steps(model, tokens, n, dtype, loss_scale=None):
     loss = None
     for _ in range(n):
         model.zero_grad(set_to_none=True)
         with torch.autocast("cuda", dtype=dtype):
             _, loss = model(tokens, tokens)
-        loss.backward()
+        (loss if loss_scale is None else loss * loss_scale).backward()
     return loss
+
+
+def time_steps(model, tokens, steps, warmup, dtype, loss_scale=None):
+    """-> (ms per step, last loss): `warmup` untimed steps, then exactly `steps` between two synchronisations."""
+    run_steps(model, tokens, warmup, dtype, loss_scale)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    loss = run_steps(model, tokens, steps, dtype, loss_scale)
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps * 1e3, float(loss.detach())
+
+
+def metric_name(workload):
+    L, d, nh, hd, f, S, B, lin_bias, alibi = WORKLOADS[workload]
+    size = workload.split("-")[1].upper()
+    return f"fwd+bwd model TFLOPs on 1 MI355X, {size} ctx{S} bs{B}; % of fp16 MFMA peak"
+
+
+def layout_name(la, lb):
+    return {(0, 1): "X.W (A k-contiguous, B k-strided)", (0, 0): "dY.W^T (both k-contiguous)",
+            (1, 1): "X^T.dY (both k-strided)", (1, 0): "A k-strided, B k-contiguous"}[(la, lb)]
+
+
+def gemm_table(by_shape, reps, workload, dtype_name):
+    """Markdown table of the instrumented GEMM calls: one row per distinct call, HIP-event time per call."""
+    rows = []
+    for key, (cnt, ms) in by_shape.items():
+        if key[0] == "group":
+            probs = key[1:]
+            flop = sum(2.0 * m * n * k for m, n, k in probs)
+            what = "grouped dW: " + " + ".join(f"{m}x{n}x{k}" for m, n, k in probs)
+            layout = layout_name(1, 1)
+        elif key[0] == "bits":
+            _, lb, m, n, k = key
+            flop, what, layout = 2.0 * m * n * k, f"{m}x{n}x{k} (ReLU sign bits)", layout_name(0, lb)
+        else:
+            la, lb, m, n, k = key
+            flop, what, layout = 2.0 * m * n * k, f"{m}x{n}x{k}", layout_name(la, lb)
+        us = ms / cnt * 1e3
+        rows.append((ms / reps, f"| {what} | {layout} | {cnt // reps} | {us:.1f} | {flop / us / 1e6:.0f} | {ms / reps:.3f} |"))
+    rows.sort(key=lambda r: -r[0])
+    head = [f"# GEMM calls of one step by shape ({workload}, {dtype_name})", "",
+            "Command (on the MI355X box, from the repository root):", "",
+            f"    python3 bench.py --workload {workload} --dtype {dtype_name} --no-cpu-baseline --no-extras --gemm-table gpurun_out/gemm_table.md",
+            "", "M x N x K of `C[M,N] = sum_k A(m,k) B(n,k)`; time = HIP events on the launch stream around the call "
+            f"(its GEMM kernel or kernels and, for a split contraction, the reduce pass), mean over {reps} instrumented steps.", "",
+            "| product (M x N x K) | operand layout | calls / step | us / call | TFLOP/s | ms / step |", "|---|---|---:|---:|---:|---:|"]
+    return "\n".join(head + [r[1] for r in rows]) + "\n"
 
 
 class GemmTimer:
@@ -175,8 +232,9 @@ def mfma_probe(dtype, device, iters=20000):
     """TFLOP/s of 256 workgroups x 8 waves issuing nothing but the GEMM step's MFMAs, per kind of operand data."""
     from tritonformer_amd import _lib
 
-    lib = _lib.load()
-    sink = torch.empty(256 * 512, dtype=torch.float32, device=device)
+    lib = _lib.load_diag()
+    wgs = torch.cuda.get_device_properties(device).multi_processor_count
+    sink = torch.empty(wgs * 512, dtype=torch.float32, device=device)
     gen = torch.Generator(device="cpu").manual_seed(0)
     kinds = {
         "all ones": torch.ones(24576),
@@ -184,17 +242,17 @@ def mfma_probe(dtype, device, iters=20000):
         "normal, std 0.02 (weights)": torch.randn(24576, generator=gen) * 0.02,
         "normal, std 1": torch.randn(24576, generator=gen),
     }
-    out = {"probe": "v_mfma_f32_32x32x16 stream of one 256x256x64 GEMM step per trip, 256 workgroups x 8 waves, "
+    out = {"probe": f"v_mfma_f32_32x32x16 stream of one 256x256x64 GEMM step per trip, {wgs} workgroups x 8 waves, "
                     "no memory traffic", "dtype": str(dtype).replace("torch.", ""), "iters": iters, "tflops": {}}
-    flops = lib.tf_probe_mfma_rate_flops(iters)
+    flops = lib.tf_diag_mfma_rate_flops(iters, wgs)
     for name, vals in kinds.items():
         ops = vals.to(dtype).to(device)
         stream = torch.cuda.current_stream().cuda_stream
-        _lib.check(lib.tf_probe_mfma_rate(stream, _lib.dtype_code(dtype), ops.data_ptr(), 100, sink.data_ptr()))
+        _lib.check(lib.tf_diag_mfma_rate(stream, _lib.dtype_code(dtype), ops.data_ptr(), 100, wgs, sink.data_ptr()))
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
-        _lib.check(lib.tf_probe_mfma_rate(stream, _lib.dtype_code(dtype), ops.data_ptr(), iters, sink.data_ptr()))
+        _lib.check(lib.tf_diag_mfma_rate(stream, _lib.dtype_code(dtype), ops.data_ptr(), iters, wgs, sink.data_ptr()))
         e1.record()
         torch.cuda.synchronize()
         out["tflops"][name] = round(flops / (e0.elapsed_time(e1) * 1e-3) / 1e12, 1)
@@ -245,6 +303,12 @@ def main():
     ap.add_argument("--dtype", default="fp16", choices=["fp16", "bf16"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-roofline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the loss-scaled / recast / other-workload timings that follow the headline")
+    ap.add_argument("--loss-scale", type=float, default=1024.0, help="scale of the `loss_scaled` extra")
+    ap.add_argument("--recast", action="store_true",
+                    help="time the headline with the fp32 weights converted to 16 bits in every forward pass")
+    ap.add_argument("--gemm-table", metavar="FILE", help="write the per-shape table of the instrumented GEMM calls there")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB streaming kernel, dst = src + 1 (known traffic: 1 GiB read, "
                          "1 GiB written) so that rocprofv3 FETCH_SIZE / WRITE_SIZE readings can be scaled")
@@ -268,21 +332,18 @@ def main():
     if args.attention_probe:
         print(json.dumps(attention_probe(args.workload, dtype, device)))
         return
+    import tritonformer_amd as T
+
     L, d, nh, hd, f, S, B, lin_bias, alibi = WORKLOADS[args.workload]
     model, tokens = make_model(args.workload, device, dtype)
+    T.set_weight_cast_cache(not args.recast)
 
-    run_steps(model, tokens, args.warmup, dtype)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    loss = run_steps(model, tokens, args.steps, dtype)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms = elapsed / args.steps * 1e3
+    ms, loss = time_steps(model, tokens, args.steps, args.warmup, dtype)
     flops = step_flops(L, d, f, S, B)
     tflops = flops / (ms * 1e-3) / 1e12
 
     out = {
-        "metric": "fwd+bwd model TFLOPs on 1 MI355X, 410M ctx2048 bs4; % of fp16 MFMA peak",
+        "metric": metric_name(args.workload),
         "value": round(tflops, 2),
         "unit": "TFLOP/s",
         "n_gpus": 1,
@@ -296,22 +357,26 @@ def main():
         "data": "synthetic",
         "config": {"workload": args.workload, "layers": L, "d_model": d, "heads": nh, "head_dim": hd, "ffn": f,
                    "seq_len": S, "global_batch": B, "vocab": VOCAB, "linear_bias": lin_bias, "alibi": alibi,
-                   "master_weights": "fp32", "autocast": args.dtype, "parallelism": "single GPU"},
+                   "master_weights": "fp32", "autocast": args.dtype, "parallelism": "single GPU",
+                   "protocol": "reference README.md:62-77: forward under autocast, loss.backward() unscaled, no optimizer",
+                   "weight_casts": "every forward pass" if args.recast else
+                                   "16-bit copies of the unchanged fp32 weights kept between steps (keyed on the "
+                                   "parameters' version counters); `recast_each_step` has the other mode"},
         "pct_of_fp16_mfma_peak": round(100.0 * tflops / PEAK_FP16_TFLOPS, 2),
         "tokens_per_s": round(B * S / (ms * 1e-3), 1),
         "step_tflop": round(flops / 1e12, 3),
-        "loss": round(float(loss.detach()), 4),
+        "loss": round(loss, 4),
     }
 
     if not args.no_roofline:
         reps = max(1, min(args.steps, 5))
         from tritonformer_amd import _lib
 
-        count0 = _lib.load().tf_gemm_launch_count()
+        count0 = _lib.load_diag().tf_diag_gemm_launch_count()
         with GemmTimer() as gt:
             run_steps(model, tokens, reps, dtype)
         calls = sum(c for c, _ in gt.by_shape.values())
-        launches = _lib.load().tf_gemm_launch_count() - count0  # kernels: a product cut along N is two
+        launches = _lib.load_diag().tf_diag_gemm_launch_count() - count0  # kernels: a product cut along N is two
         total_ms = sum(t for _, t in gt.by_shape.values())
         gflops = gemm_flops(L, d, f, S, B) * reps
         achieved = gflops / (total_ms * 1e-3) / 1e12
@@ -332,6 +397,41 @@ def main():
                         "run after the timed ones; the event time of a call covers its GEMM kernel(s) and, for a split contraction, "
                         "the reduce kernel; launches = GEMM kernels counted by the library",
         }
+        if args.gemm_table:
+            with open(args.gemm_table, "w") as fh:
+                fh.write(gemm_table(gt.by_shape, reps, args.workload, args.dtype))
+    if not args.no_extras:
+        k, w = max(3, args.steps // 2), 2
+        ms_s, loss_s = time_steps(model, tokens, k, w, dtype, loss_scale=args.loss_scale)
+        out["loss_scaled"] = {"scale": args.loss_scale, "ms_per_step": round(ms_s, 3), "steps": k,
+                              "value": round(flops / (ms_s * 1e-3) / 1e12, 2), "loss": round(loss_s, 4)}
+        if not args.recast:
+            T.set_weight_cast_cache(False)
+            ms_r, _ = time_steps(model, tokens, k, w, dtype)
+            T.set_weight_cast_cache(True)
+            out["recast_each_step"] = {"ms_per_step": round(ms_r, 3), "steps": k,
+                                       "value": round(flops / (ms_r * 1e-3) / 1e12, 2)}
+        del model
+        others = []
+        for name, dts in (("gpt2-160m-ctx2048-bs8", ["fp16"]), ("gpt2-410m-ctx2048-bs4", ["fp16"]),
+                          ("gpt2-840m-alibi-ctx4096-bs1", ["fp16"]), ("gpt2-1.4b-ctx2048-bs2", ["fp16", "bf16"])):
+            if name == args.workload:
+                continue
+            torch.cuda.empty_cache()
+            m2, tok2 = make_model(name, device, dtype)
+            L2, d2, _, _, f2, S2, B2, _, _ = WORKLOADS[name]
+            for dn in dts:
+                T.clear_weight_cast_cache()
+                ms2, loss2 = time_steps(m2, tok2, 5, 2, torch.float16 if dn == "fp16" else torch.bfloat16)
+                fl2 = step_flops(L2, d2, f2, S2, B2)
+                others.append({"workload": name, "dtype": dn, "ms_per_step": round(ms2, 3), "steps": 5,
+                               "value": round(fl2 / (ms2 * 1e-3) / 1e12, 2),
+                               "pct_of_fp16_mfma_peak": round(100.0 * fl2 / (ms2 * 1e-3) / 1e12 / PEAK_FP16_TFLOPS, 2),
+                               "loss": round(loss2, 4)})
+            del m2, tok2
+        T.clear_weight_cast_cache()
+        torch.cuda.empty_cache()
+        out["workloads"] = others
     if args.calibrate_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device=device).normal_()
         dst = torch.empty_like(src)

@@ -9,7 +9,9 @@
  *
  * Conventions
  *  - every pointer is a DEVICE pointer unless said otherwise; the library
- *    never allocates, frees, retains or synchronises; work is enqueued on
+ *    never allocates, frees, retains or synchronises; it reads no environment
+ *    variable and keeps no state between calls beyond the device's CU / XCD
+ *    counts; work is enqueued on
  *    `stream` (a hipStream_t passed as void*, NULL = the null stream);
  *  - strides and leading dimensions are in ELEMENTS, sizes in elements;
  *  - `dtype`: TF_F16 / TF_BF16 for the 16-bit paths, TF_F32 only where stated;
@@ -46,6 +48,13 @@ enum tf_op_layout { TF_OP_KMAJOR = 0, TF_OP_KMINOR = 1 };
 
 const char* tf_status_string(int status);
 int tf_version(void);
+/* Hash of the source files this binary was built from ("" for a build that did not record
+ * one); the Python loader refuses a library whose hash differs from the sources beside it. */
+const char* tf_source_hash(void);
+/* Compute units and XCDs of the current HIP device as the library sees them (read from the
+ * runtime once per device; tile choice and the workgroup-id remap of the GEMM kernels use them).
+ * The reference has no counterpart: Triton reads the device through its own driver layer. */
+int tf_device_info(int* cus, int* xcds);
 
 /* ---- dense contractions (fp16/bf16 MFMA, fp32 accumulate) --------------- */
 
@@ -137,29 +146,6 @@ int tf_gemm_group(void* stream, int dtype, int out_dtype, int layout_a, int layo
                   const tf_gemm_problem* problems, void* workspace, int64_t workspace_bytes);
 int64_t tf_gemm_group_workspace_bytes(int layout_a, int layout_b, int count,
                                       const tf_gemm_problem* problems);
-/* Diagnostic: number of GEMM kernels launched by this library since it was loaded (the reduce
- * passes of split contractions are not counted; one tf_gemm* call may launch two kernels when
- * the product is cut along N).  No counterpart in the reference. */
-int64_t tf_gemm_launch_count(void);
-/* Diagnostic, no counterpart in the reference (whose Triton autotuner picks
- * tiles per shape, kernels/gemm.py:15-79): force tile configuration `cfg`
- * (-1 = automatic) and contraction split `splits` (0 = automatic) for all
- * later tf_gemm / tf_gemm_workspace_bytes calls of this process. */
-int tf_gemm_tune(int cfg, int splits);
-/* Diagnostic: bit 0 disables the XCD-aware workgroup remap; bit 3 skips the
- * result write-out (WRONG results: it exists to time the main loop alone); bit 6
- * disables the cut of a nearly empty last round of tiles into a split-contraction tail. */
-int tf_gemm_debug_flags(int flags);
-
-/* Diagnostic, no counterpart in the reference: the MFMA instruction stream of the
- * 256x256x64 GEMM step alone (one workgroup per CU, 8 waves, no memory traffic),
- * `iters` steps per workgroup, operands taken once from `operands` (8*6*64*8 = 24576
- * elements of `dtype`, device memory); `sink`: 256*512 floats.  Time the call and divide
- * tf_probe_mfma_rate_flops(iters) by it: the sustained rate depends on the operand
- * values (the clock drops under the switching activity of random data). */
-int tf_probe_mfma_rate(void* stream, int dtype, const void* operands, int iters, float* sink);
-int64_t tf_probe_mfma_rate_flops(int iters);
-
 /* Causal flash attention forward.  q, k, v: logical (B, nh, S, hd) sharing the
  * element strides {sb, sh, ss}; o: the same logical shape with its own strides
  * {osb, osh, oss}; unit stride along hd everywhere.  (The reference passes q's
@@ -172,7 +158,11 @@ int64_t tf_probe_mfma_rate_flops(int iters);
  * (kernels/biased_attention.py:101-106); -inf entries are allowed.
  * Replaces flash_wrapper_fwd (kernels/attention.py:171-217) and
  * flash_wrapper_fwd_attn_bias (kernels/biased_attention.py:188-245).
- * Preconditions (as the reference asserts): hd in {32,64,128}; S % 64 == 0. */
+ * Preconditions: hd in {32,64,128} (as the reference asserts); S % 64 == 0.  The reference
+ * asserts S % 64 == 0 too, except at hd = 128, where its 32-row blocks admit S % 32 == 0
+ * (kernels/attention.py:177-183); a caller with such a length continues q, k, v with 32 rows
+ * of zeros (under the causal mask no real query sees them) and drops the added output rows,
+ * as the Python launcher of this package does. */
 int tf_attn_fwd(void* stream, int dtype, int64_t B, int64_t nh, int64_t S, int64_t hd,
                 const void* q, const void* k, const void* v, void* o,
                 int64_t sb, int64_t sh, int64_t ss, int64_t osb, int64_t osh, int64_t oss,
@@ -333,10 +323,11 @@ int tf_cross_entropy_bwd(void* stream, int dtype, int64_t rows, int64_t V,
                          const int64_t* labels, const float* lse, const void* gout, int64_t gout_stride,
                          void* dlogits, int64_t ldd, int64_t outer_stride_d);
 
-/* out[c] = sum_r x[r, c] with fp32 accumulation (bias gradient).
+/* out[c] = sum_r x[r, c] with fp32 accumulation (bias gradient); `out` has out_dtype:
+ * `dtype`, or TF_F32 (the gradient of an fp32 master bias, stored unrounded).
  * Replaces unbroadcast_leading (kernels/reductions.py:97-122, two-stage with
  * _unbroadcast :57-63).  partial: fp32 scratch of tf_colsum_partial_bytes(). */
-int tf_colsum(void* stream, int dtype, int64_t rows, int64_t cols,
+int tf_colsum(void* stream, int dtype, int out_dtype, int64_t rows, int64_t cols,
               const void* x, int64_t ldx, void* out,
               float* partial, int64_t partial_bytes);
 int64_t tf_colsum_partial_bytes(int64_t rows, int64_t cols);

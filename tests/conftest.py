@@ -18,8 +18,9 @@ def built_artifacts():
     """Load what is built; build only if nothing is (hipcc cross-compiles without a GPU)."""
     from tritonformer_amd import _build, _lib
 
-    if not os.path.exists(_lib.LIB_PATH):
+    if not (os.path.exists(_lib.LIB_PATH) and os.path.exists(_lib.DIAG_LIB_PATH)):
         _build.build_library(verbose=False)
+    _lib.load()   # refuses a library built from other sources than the ones in the tree
     ref_so = os.path.join(ROOT, "oracle", "libref_ops.so")
     if not os.path.exists(ref_so):
         subprocess.run(["make", "-C", os.path.join(ROOT, "oracle")], check=True, capture_output=True)

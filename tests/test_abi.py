@@ -13,10 +13,11 @@ from tritonformer_amd import _lib
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "tritonformer_amd.h")
+DIAG_HEADER = os.path.join(ROOT, "include", "tritonformer_amd_diag.h")
 
 
-def declared_functions():
-    text = open(HEADER).read()
+def declared_functions(header=HEADER):
+    text = open(header).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(tf_[a-z0-9_]+)\s*\(", text)))
 
@@ -38,6 +39,38 @@ def test_library_exports_every_declared_symbol():
 
 def test_binding_table_matches_header():
     assert sorted(_lib.SIGNATURES) == declared_functions()
+
+
+def test_diagnostics_are_declared_apart_and_exported():
+    """Diagnostics have a header of their own; the product header names none of them, the two
+    libraries export what that header declares, and the binding table mirrors it."""
+    names = declared_functions(DIAG_HEADER)
+    assert names and all(n.startswith("tf_diag_") for n in names)
+    assert not [n for n in declared_functions() if "diag" in n or "probe" in n or "tune" in n or "debug" in n]
+    assert sorted(_lib.DIAG_SIGNATURES) == names
+    libs = {"main": ctypes.CDLL(_lib.LIB_PATH), "diag": ctypes.CDLL(_lib.DIAG_LIB_PATH)}
+    for name, (where, _, _) in _lib.DIAG_SIGNATURES.items():
+        assert hasattr(libs[where], name), f"{name} not exported by the {where} library"
+
+
+def test_library_reads_no_environment_and_reports_its_sources():
+    """No getenv in the product sources (tile choice cannot be switched from outside the call), and
+    the binary carries the hash of the sources it was built from."""
+    from tritonformer_amd import _build
+
+    csrc = os.path.join(ROOT, "tritonformer_amd", "csrc")
+    for f in os.listdir(csrc):
+        if f.endswith((".hip", ".h")):
+            assert "getenv" not in open(os.path.join(csrc, f)).read(), f
+    assert _lib.load().tf_source_hash().decode() == _build.source_hash()
+
+
+def test_device_info_has_a_fallback_without_a_gpu():
+    lib = _lib.load()
+    cus, xcds = ctypes.c_int(0), ctypes.c_int(0)
+    assert lib.tf_device_info(ctypes.byref(cus), ctypes.byref(xcds)) == 0
+    assert cus.value > 0 and xcds.value > 0 and cus.value % xcds.value == 0
+    assert lib.tf_device_info(None, None) == -1
 
 
 def test_status_strings():
@@ -105,12 +138,20 @@ def test_gemm_rejects_bad_arguments():
     assert lib.tf_cast_pack(None, 2, 0, 3, 0, 8, ptrs, 8, FAKE, 24) == 0           # nothing to do
 
 
-def test_probe_rejects_bad_arguments():
-    lib = _lib.load()
-    assert lib.tf_probe_mfma_rate(None, 0, None, 10, FAKE) == -1
-    assert lib.tf_probe_mfma_rate(None, 0, FAKE, 0, FAKE) == -1
-    assert lib.tf_probe_mfma_rate(None, 2, FAKE, 10, FAKE) == -2
-    assert lib.tf_probe_mfma_rate_flops(10) == 10 * 256 * 2 * 256 * 256 * 64
+def test_diagnostics_reject_bad_arguments():
+    d = _lib.load_diag()
+    assert d.tf_diag_mfma_rate(None, 0, None, 10, 256, FAKE) == -1
+    assert d.tf_diag_mfma_rate(None, 0, FAKE, 0, 256, FAKE) == -1
+    assert d.tf_diag_mfma_rate(None, 0, FAKE, 10, 0, FAKE) == -1
+    assert d.tf_diag_mfma_rate(None, 2, FAKE, 10, 256, FAKE) == -2
+    assert d.tf_diag_mfma_rate_flops(10, 256) == 10 * 256 * 2 * 256 * 256 * 64
+    g = lambda cfg, splits, flags: d.tf_diag_gemm(None, cfg, splits, flags, 0, 0, 0, 1, 64, 64, 64, None, 64, FAKE, 64,
+                                                  FAKE, 64, None, 0, None, 0)
+    assert g(99, 0, 0) == -1 and g(2, -1, 0) == -1 and g(2, 0, 8) == -1   # unknown cfg, negative split, refused flag bit
+    assert g(2, 0, 0) == -1                                               # then the ordinary checks (null A)
+    # a forced split is priced by the size query
+    assert d.tf_diag_gemm_workspace_bytes(2, 4, 256, 256, 1024) == 4 * 256 * 256 * 4
+    assert d.tf_diag_gemm_workspace_bytes(2, 1, 256, 256, 1024) == 0
 
 
 def test_embedding_rejects_bad_arguments():
@@ -202,7 +243,8 @@ def test_row_kernels_reject_bad_arguments():
     assert lib.tf_cross_entropy_fwd(None, 2, 4, 64, FAKE, 64, 0, 0, FAKE, FAKE, FAKE) == -2
     assert lib.tf_cross_entropy_bwd(None, 0, 4, 64, FAKE, 32, 0, 0, FAKE, FAKE, FAKE, 1, FAKE, 64, 0) == -1
     assert lib.tf_cross_entropy_fwd(None, 0, 6, 64, FAKE, 64, 3, 100, FAKE, FAKE, FAKE) == -1   # groups overlap
-    assert lib.tf_colsum(None, 0, 16, 64, FAKE, 64, FAKE, None, 0) == -5
+    assert lib.tf_colsum(None, 0, 0, 16, 64, FAKE, 64, FAKE, None, 0) == -5
+    assert lib.tf_colsum(None, 0, 1, 16, 64, FAKE, 64, FAKE, FAKE, 1 << 20) == -2   # bf16 sums of fp16 input
     assert lib.tf_relu_mask(None, 0, 4, 64, None, 64, FAKE, 64, FAKE, 64) == -1
     # empty inputs are accepted and launch nothing
     assert lib.tf_softmax_fwd(None, 0, 0, 64, FAKE, 64, FAKE, 64) == 0

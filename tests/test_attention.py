@@ -26,6 +26,10 @@ DIMS = [(int(b), int(nh), int(sq), int(hd))
         for sq in 64 * rng.randint(1, 12, size=NUM_TEST)
         for hd in rng.choice([32, 64], size=1)]
 EDGE = [(1, 1, 64, 64), (1, 2, 64, 32), (2, 3, 128, 64), (1, 2, 192, 128), (1, 4, 320, 128), (2, 2, 1024, 64)]
+# the upper ends of the reference's draws (test_attention.py:66-73: nh < 32, S = 64 * [1, 32), B < 4)
+UPPER = [(1, 31, 1984, 64), (3, 5, 1984, 32)]
+# head_dim 128 with S = 32 (mod 64): lengths the reference's 32-row blocks admit (kernels/attention.py:177-183)
+HD128_S32 = [(1, 2, 32, 128), (2, 3, 96, 128), (1, 2, 160, 128)]
 
 
 def make_qkv(dims, dtype, dev, seed=0, strided=True):
@@ -61,9 +65,19 @@ def run_case(dims, dtype, dev, bias=None, strided=True, seed=0, kernel_bias=None
     return o, qd, kd, vd
 
 
-@pytest.mark.parametrize("dims", DIMS + EDGE)
+@pytest.mark.parametrize("dims", DIMS + EDGE + UPPER)
 def test_attn_fwd_bwd(dims, dev):
     run_case(dims, torch.float16, dev)
+
+
+@pytest.mark.parametrize("dims", HD128_S32)
+@pytest.mark.parametrize("strided", [True, False])
+def test_attn_head_dim_128_takes_multiples_of_32(dims, strided, dev):
+    run_case(dims, torch.float16, dev, strided=strided)
+    run_case(dims, torch.bfloat16, dev, strided=strided, seed=1)
+    with pytest.raises(ValueError):     # 64-wide heads keep the reference's multiple-of-64 rule
+        q = torch.zeros(1, 2, dims[2], 64, dtype=torch.float16, device=dev)
+        T.fast_causal_attention.apply(q, q, q)
 
 
 @pytest.mark.parametrize("dims", [(1, 2, 128, 64), (2, 3, 256, 32), (1, 2, 192, 128)])

@@ -119,3 +119,47 @@ def test_wrapper_preconditions():
         K.layernorm_fwd(torch.zeros(1, 4, 8), torch.ones(8), torch.zeros(8), 1e-5)
     with pytest.raises(ValueError):
         K.layernorm_fwd(torch.zeros(4, 8, dtype=h), torch.ones(8, dtype=h), torch.zeros(8, dtype=h), 1e-5)
+
+
+def test_weight_cast_cache_invalidation():
+    """The cache of 16-bit weight copies returns the stored tensor only while the very same parameter
+    objects hold the same storage at the same version; in-place updates, a new storage, another
+    parameter object or another dtype convert again.  (Host logic: runs on CPU tensors.)"""
+    import torch
+    from tritonformer_amd import _amp
+
+    calls = []
+
+    def convert(ws, dt):
+        calls.append(1)
+        return torch.cat([w.to(dt) for w in ws], dim=1)
+
+    a, b = torch.nn.Parameter(torch.randn(4, 3)), torch.nn.Parameter(torch.randn(4, 5))
+    assert not _amp.weight_cast_cache_enabled()
+    _amp.cached_conversion([a, b], torch.float16, convert)
+    _amp.cached_conversion([a, b], torch.float16, convert)
+    assert len(calls) == 2                               # off by default: every call converts
+    _amp.set_weight_cast_cache(True)
+    try:
+        first = _amp.cached_conversion([a, b], torch.float16, convert)
+        assert _amp.cached_conversion([a, b], torch.float16, convert) is first and len(calls) == 3
+        with torch.no_grad():
+            a.add_(1.0)                                  # in-place update: version counter moves
+        second = _amp.cached_conversion([a, b], torch.float16, convert)
+        assert second is not first and len(calls) == 4
+        assert torch.equal(second, torch.cat([a.half(), b.half()], dim=1))
+        torch.autograd.graph.increment_version(b)        # what the fused AdamW does after its kernel
+        assert _amp.cached_conversion([a, b], torch.float16, convert) is not second and len(calls) == 5
+        a.data = torch.randn(4, 3)                       # new storage
+        _amp.cached_conversion([a, b], torch.float16, convert)
+        assert len(calls) == 6
+        _amp.cached_conversion([a, b], torch.bfloat16, convert)     # another dtype: its own entry
+        assert len(calls) == 7
+        _amp.cached_conversion([a.detach(), b.detach()], torch.float16, convert)   # not parameters: never cached
+        _amp.cached_conversion([a.detach(), b.detach()], torch.float16, convert)
+        assert len(calls) == 9
+        _amp.clear_weight_cast_cache()
+        _amp.cached_conversion([a, b], torch.float16, convert)
+        assert len(calls) == 10
+    finally:
+        _amp.set_weight_cast_cache(False)

@@ -16,7 +16,8 @@ rng = np.random.RandomState(0)
 DIMS = [(int(b), int(s), int(d)) for b in rng.randint(1, 16, size=NUM_TEST) for s in rng.randint(64, 512, size=1)
         for d in rng.randint(64, 1024, size=NUM_TEST)]
 EDGE = [(1, 1, 8), (1, 3, 7), (2, 64, 768), (3, 77, 333), (1, 130, 1024), (2, 33, 2048), (1, 17, 4096), (1, 9, 5000),
-        (1, 5, 8192)]
+        (1, 5, 8192),
+        (31, 1023, 1021), (31, 64, 1016)]  # upper end of the reference's draws (test_layernorm.py:35-37)
 
 
 def run_case(dims, dtype, dev):

@@ -26,6 +26,8 @@ RANDOM_DIMS = [(int(b), int(m), int(n), int(k))
                for k in rng.randint(64, 1536, size=1)]
 EDGE_DIMS = [(1, 1, 8, 8), (1, 64, 64, 64), (2, 77, 333, 129), (3, 130, 264, 520), (1, 257, 1024, 72),
              (2, 512, 768, 3072), (1, 300, 4096, 1024)]
+# the upper end of the reference's draws (test_linear.py:36-41: B < 32, M, N, K < 4096), ragged
+UPPER_DIMS = [(31, 4001, 4093, 3999)]
 VARIANTS = {
     "nobias": (T.linear_no_bias, False, False),
     "bias": (T.linear_bias, True, False),
@@ -44,18 +46,22 @@ def make(dims, dtype, dev, seed):
     return x, w, bias, dy
 
 
-def run_case(dims, variant, dtype, dev, seed=0):
+def run_case(dims, variant, dtype, dev, seed=0, oracle_on_gpu=False):
+    """``oracle_on_gpu``: the fp32 oracle expressions evaluated on the GPU (rocBLAS fp32) instead
+    of the CPU, for cases whose CPU time would run to minutes."""
     fn, use_bias, relu = VARIANTS[variant]
     x, w, bias, dy = make(dims, dtype, dev, seed)
     xd, wd, bd = (t.to(dev).requires_grad_(True) for t in (x, w, bias))
     y = fn.apply(xd, wd, bd) if use_bias else fn.apply(xd, wd)
     y.backward(dy.to(dev))
+    if oracle_on_gpu:
+        x, w, bias, dy = (t.to(dev) for t in (x, w, bias, dy))
     y_ref = R.linear(x, w, bias if use_bias else None, relu)
     assert_close(y, y_ref, dtype, f"{variant} y {dims}")
     # the ReLU gradient mask is the sign of the kernel's own rounded output (as in the
     # reference, linear.py:62): on a pre-activation within rounding of zero fp32 and
     # 16-bit math may disagree, which is not an error of the backward kernels
-    act = y.detach().cpu() if relu else None
+    act = (y.detach() if oracle_on_gpu else y.detach().cpu()) if relu else None
     dx_ref, dw_ref, db_ref = R.linear_bwd(x, w, dy, act=act, with_bias=use_bias)
     big = dims[0] * dims[1]  # contraction length of dW: rounding noise grows like sqrt
     assert_close(xd.grad, dx_ref, dtype, f"{variant} dx {dims}")
@@ -70,6 +76,17 @@ def run_case(dims, variant, dtype, dev, seed=0):
 @pytest.mark.parametrize("variant", ["nobias", "bias"])
 def test_linear_fwd_bwd(dims, variant, dev):
     run_case(dims, variant, torch.float16, dev)
+
+
+@pytest.mark.parametrize("dims", UPPER_DIMS)
+@pytest.mark.parametrize("variant", ["bias", "relu"])
+def test_linear_upper_end_of_reference_range(dims, variant, dev):
+    run_case(dims, variant, torch.float16, dev, oracle_on_gpu=True)
+
+
+def test_linear_large_ragged_against_cpu_oracle(dev):
+    """M, N, K near the top of the reference's range, ragged, with the oracle on the CPU."""
+    run_case((3, 3999, 4093, 4001), "biasrelu", torch.float16, dev)
 
 
 @pytest.mark.parametrize("dims", EDGE_DIMS + RANDOM_DIMS[:3])
@@ -177,6 +194,93 @@ def test_logits_projection_shape(dev):
     dx, dw, _ = R.linear_bwd(x.detach(), w.detach(), dy)
     assert_close(x.grad, dx, name="dx", atol=2e-2)
     assert rel_l2(w.grad, dw) < 1e-3
+
+
+@pytest.mark.parametrize("d_in,f,d_out", [(64, 128, 72), (128, 256, 200), (256, 512, 64), (72, 128, 64)])
+@pytest.mark.parametrize("use_bias", [False, True])
+def test_fused_mlp_with_different_input_and_output_widths(d_in, f, d_out, use_bias, dev):
+    """x (.., d_in) W1 (d_in, f) W2 (f, d_out) with d_out != d_in: the forward product (contraction
+    over d_in) may keep the ReLU mask as sign bits while the backward product dH = dY W2^T
+    (contraction over d_out) misses the preconditions of the kernel that reads them (d_out not a
+    multiple of 64); the backward then masks with the saved activation.  Must equal the two
+    Functions bit for bit either way."""
+    g = torch.Generator().manual_seed(13)
+    x = torch.randn(2, 96, d_in, generator=g).half().to(dev)
+    w1 = (torch.randn(d_in, f, generator=g) / d_in ** 0.5).half().to(dev)
+    w2 = (torch.randn(f, d_out, generator=g) / f ** 0.5).half().to(dev)
+    b1 = torch.randn(f, generator=g).half().to(dev) if use_bias else None
+    b2 = torch.randn(d_out, generator=g).half().to(dev) if use_bias else None
+    dy = torch.randn(2, 96, d_out, generator=g).half().to(dev)
+    a = [t.clone().requires_grad_(True) if t is not None else None for t in (x, w1, b1, w2, b2)]
+    ya = T.mlp_fused_relu.apply(*a)
+    ya.backward(dy)
+    c = [t.clone().requires_grad_(True) if t is not None else None for t in (x, w1, b1, w2, b2)]
+    if use_bias:
+        yb = T.linear_bias.apply(T.linear_fused_bias_relu.apply(c[0], c[1], c[2]), c[3], c[4])
+    else:
+        yb = T.linear_no_bias.apply(T.linear_fused_relu.apply(c[0], c[1]), c[3])
+    yb.backward(dy)
+    assert torch.equal(ya, yb)
+    for ta, tb in zip(a, c):
+        if ta is not None:
+            assert torch.equal(ta.grad, tb.grad)
+    hidden = R.linear(x.cpu(), w1.cpu(), b1.cpu() if use_bias else None, True).half()
+    assert_close(ya, R.linear(hidden, w2.cpu(), b2.cpu() if use_bias else None), name="mlp y", atol=2e-2)
+
+
+def test_bias_gradient_of_fp32_master_bias_is_unrounded(dev):
+    """Under autocast an fp32 bias gets the fp32 column sums themselves, not a 16-bit rounding of
+    them cast back: the sums of 16384 rows of values near 1 would lose 3 digits in fp16."""
+    g = torch.Generator().manual_seed(17)
+    x = torch.randn(8, 2048, 64, generator=g).to(dev).requires_grad_(True)
+    w = (torch.randn(64, 128, generator=g) / 8).to(dev).requires_grad_(True)
+    b = torch.zeros(128, device=dev, requires_grad=True)
+    dy = (1.0 + 0.1 * torch.randn(8, 2048, 128, generator=g)).half()
+    with torch.autocast("cuda", dtype=torch.float16):
+        y = T.linear_bias.apply(x, w, b)
+    y.backward(dy.to(dev))
+    want = dy.double().sum((0, 1))
+    assert b.grad.dtype == torch.float32
+    assert (b.grad.cpu().double() - want).abs().max() <= 2e-6 * want.abs().max()   # fp16 would be off by ~8
+    with torch.autocast("cuda", dtype=torch.float16):
+        y = T.mlp_fused_relu.apply(x, w, b, w.detach().T.contiguous().requires_grad_(True), None)
+    b.grad = None
+    y.sum().backward()
+    assert b.grad.dtype == torch.float32 and torch.isfinite(b.grad).all()
+
+
+@pytest.mark.parametrize("layouts", ["fwd", "dx", "dw"])
+def test_every_tile_configuration_gives_the_same_product(layouts, dev):
+    """The diagnostic entry point imposes each tile configuration in turn on one product that all
+    of them can take: an unsplit contraction sums the same 64-wide steps in the same order whatever
+    the tile shape, so the results are equal bit for bit; a split one differs in fp32 summation
+    order only.  Also with the XCD remap of workgroup ids switched off."""
+    from tritonformer_amd import _lib
+
+    d = _lib.load_diag()
+    g = torch.Generator().manual_seed(23)
+    M, N, K = 640, 768, 512
+    la, lb = {"fwd": (0, 1), "dx": (0, 0), "dw": (1, 1)}[layouts]
+    a = torch.randn((M, K) if la == 0 else (K, M), generator=g).half().to(dev)
+    b = (torch.randn((N, K) if lb == 0 else (K, N), generator=g) / K ** 0.5).half().to(dev)
+    a32, b32 = (a.float() if la == 0 else a.float().T), (b.float() if lb == 0 else b.float().T)
+    want = a32 @ b32.T
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def run(cfg, splits, flags):
+        out = torch.empty((M, N), dtype=torch.float16, device=dev)
+        nb = d.tf_diag_gemm_workspace_bytes(cfg, splits, M, N, K)
+        ws = torch.empty(max(nb, 16), dtype=torch.uint8, device=dev)
+        _lib.check(d.tf_diag_gemm(stream, cfg, splits, flags, 0, 0, la, lb, M, N, K, a.data_ptr(), a.stride(0),
+                                  b.data_ptr(), b.stride(0), out.data_ptr(), N, None, 0, ws.data_ptr(), nb))
+        return out
+
+    base = run(-1, 0, 0)
+    assert_close(base, want, name=f"{layouts} auto")
+    for cfg in range(6):
+        assert torch.equal(run(cfg, 1, 0), base), f"cfg {cfg}"
+        assert torch.equal(run(cfg, 1, 1), base), f"cfg {cfg} without the XCD remap"
+        assert rel_l2(run(cfg, 4, 0), base) < 1e-3, f"cfg {cfg} split 4"
 
 
 @pytest.mark.parametrize("dims,use_bias", [((2, 128, 256, 1024), False), ((3, 77, 136, 264), True),

@@ -272,3 +272,117 @@ def test_model_golden_fixture():
     assert abs(got["loss"] - want["loss"]) <= 1e-5 * abs(want["loss"])
     for name, norm in want["grad_norms"].items():
         assert abs(got["grad_norms"][name] - norm) <= 1e-3 * norm + 1e-9, name
+
+
+# --------------------------------------------------------------------------- block wiring of the oracle model
+def _random_norm_params(model):
+    """LayerNorm gamma / beta away from (1, 0): with the initial values a LayerNorm applied
+    twice equals one applied once, and a misplaced one would go unnoticed."""
+    g = torch.Generator().manual_seed(5)
+    for name, p in model.named_parameters():
+        if "layernorm" in name:
+            p.data = (torch.rand(p.shape, generator=g) + 0.5) if name.endswith("weight") else torch.randn(p.shape, generator=g) * 0.3
+
+
+def _branch_outputs(model, ids):
+    """logits plus what each attention / MLP module returned, in call order."""
+    seen, hooks = [], []
+    for layer in model.layer_list:
+        hooks.append(layer.attention.register_forward_hook(lambda m, i, o: seen.append(("attn", o.detach()))))
+        hooks.append(layer.mlp.register_forward_hook(lambda m, i, o: seen.append(("mlp", o.detach()))))
+    with torch.no_grad():
+        logits = model(ids, None)
+    for h in hooks:
+        h.remove()
+    return logits, seen
+
+
+@pytest.mark.parametrize("alibi", [False, True])
+def test_model_wiring_is_pre_ln_with_both_residuals(alibi):
+    """What reference transformer.py:238-251, 311-331 fixes, checked on quantities a wrong wiring
+    changes: (a) the residual stream is the embedding plus every branch output, and the logits
+    are final_layernorm(stream) @ W_out -- a dropped residual, a branch added to the normalised
+    input or a LayerNorm on the stream (post-LN) fails it; (b) each branch reads a LayerNorm of
+    the stream, so scaling the embeddings by c leaves the first attention output unchanged, and
+    the first MLP output too once the attention output is silenced; (c) with both output
+    projections zero the logits are LN_f(embedding) @ W_out in closed form."""
+    cfg = R.RefConfig(97, 32, 24, 4, 8, 64, 3, True, alibi)
+    torch.manual_seed(3)
+    model = R.RefTransformer(cfg)
+    model.logits_out.weight.data.normal_(0.0, 0.3)
+    _random_norm_params(model)
+    for name, p in model.named_parameters():   # biases away from zero as well
+        if name.endswith("bias") and "layernorm" not in name:
+            p.data.normal_(0.0, 0.1)
+    ids = torch.randint(0, 97, (2, 24))
+
+    def embed(m):
+        x = m.embed_tokens.weight[ids]
+        if m.embed_positions is not None:
+            x = x + m.embed_positions.weight[torch.arange(24)][None]
+        return x.detach()
+
+    def head(m, x):
+        f = m.final_layernorm
+        return F.layer_norm(x, (32,), f.weight, f.bias, f.eps) @ m.logits_out.weight
+
+    # (a) stream = embedding + all branch outputs
+    logits, seen = _branch_outputs(model, ids)
+    assert [k for k, _ in seen] == ["attn", "mlp"] * 3
+    stream = embed(model) + sum(o for _, o in seen)
+    close(logits, head(model, stream).detach())
+    # the branch inputs are LayerNorms of the running stream: recompute branch by branch
+    x = embed(model)
+    bias = model.attn_bias
+    for li, layer in enumerate(model.layer_list):
+        ln1, ln2 = layer.input_layernorm, layer.post_attention_layernorm
+        a = layer.attention(F.layer_norm(x, (32,), ln1.weight, ln1.bias, ln1.eps), bias).detach()
+        close(a, seen[2 * li][1])
+        x = x + a
+        m = layer.mlp(F.layer_norm(x, (32,), ln2.weight, ln2.bias, ln2.eps)).detach()
+        close(m, seen[2 * li + 1][1])
+        x = x + m
+
+    # (b) pre-LN: branches do not see the scale of the stream
+    scaled = R.RefTransformer(cfg)
+    scaled.load_state_dict(model.state_dict())
+    scaled.embed_tokens.weight.data *= 7.0
+    if scaled.embed_positions is not None:
+        scaled.embed_positions.weight.data *= 7.0
+    for m in (model, scaled):
+        for layer in m.layer_list:
+            layer.input_layernorm.eps = layer.post_attention_layernorm.eps = 0.0   # exact scale invariance
+    _, seen1 = _branch_outputs(model, ids)
+    _, seen7 = _branch_outputs(scaled, ids)
+    close(seen7[0][1], seen1[0][1], tol=1e-4)                    # first attention output: unchanged
+    assert (seen7[1][1] - seen1[1][1]).abs().max() > 1e-3        # first MLP saw stream = c x + a: changed
+    for m in (model, scaled):
+        m.layer_list[0].attention.out_proj.weight.data.zero_()
+    _, seen1 = _branch_outputs(model, ids)
+    _, seen7 = _branch_outputs(scaled, ids)
+    assert seen1[0][1].abs().max() == 0
+    close(seen7[1][1], seen1[1][1], tol=1e-4)                    # ... now the first MLP output is unchanged too
+
+    # (c) both output projections zero: logits = LN_f(embedding) @ W_out
+    for layer in model.layer_list:
+        layer.attention.out_proj.weight.data.zero_()
+        layer.mlp.dense_4h_to_h.weight.data.zero_()
+        layer.mlp.dense_4h_to_h.bias.data.zero_()
+    with torch.no_grad():
+        logits0 = model(ids, None)
+    close(logits0, head(model, embed(model)).detach())
+
+
+def test_model_loss_is_the_shifted_mean():
+    """reference transformer.py:332-343: row (b, s), s < S-1, is scored against labels[b, s+1];
+    the loss is the mean over the B*(S-1) rows."""
+    cfg = R.RefConfig(53, 16, 12, 2, 8, 32, 1, False, False)
+    torch.manual_seed(4)
+    model = R.RefTransformer(cfg)
+    model.logits_out.weight.data.normal_(0.0, 0.5)
+    ids, labels = torch.randint(0, 53, (3, 12)), torch.randint(0, 53, (3, 12))
+    with torch.no_grad():
+        logits, loss = model(ids, labels)
+    lp = torch.log_softmax(logits.double(), -1)
+    want = -sum(lp[b, s, labels[b, s + 1]] for b in range(3) for s in range(11)) / 33
+    assert abs(loss.item() - want.item()) < 1e-5

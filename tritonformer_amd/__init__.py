@@ -19,3 +19,4 @@ from .linear import LinearNoBiasReLU as linear_fused_relu
 from .linear import MLPReLU as mlp_fused_relu
 from .linear import PackedLinearNoBias as linear_no_bias_packed
 from .softmax import Softmax
+from ._amp import clear_weight_cast_cache, set_weight_cast_cache, weight_cast_cache_enabled

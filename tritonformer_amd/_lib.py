@@ -21,6 +21,8 @@ _vp, _i, _i64, _f = _c.c_void_p, _c.c_int, _c.c_int64, _c.c_float
 SIGNATURES = {
     "tf_status_string": (_c.c_char_p, [_i]),
     "tf_version": (_i, []),
+    "tf_source_hash": (_c.c_char_p, []),
+    "tf_device_info": (_i, [_vp, _vp]),
     "tf_gemm": (_i, [_vp, _i, _i, _i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i, _vp, _i64]),
     "tf_gemm_out": (_i, [_vp, _i, _i, _i, _i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i, _vp, _i64,
                          _vp, _i64]),
@@ -33,14 +35,9 @@ SIGNATURES = {
     "tf_embedding_bwd_workspace_bytes": (_i64, [_i64]),
     "tf_embedding_bwd": (_i, [_vp, _i, _i, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64]),
     "tf_adamw_step": (_i, [_vp, _i, _i, _vp, _f, _f, _f, _f, _f, _i64]),
-    "tf_probe_mfma_rate": (_i, [_vp, _i, _vp, _i, _vp]),
-    "tf_probe_mfma_rate_flops": (_i64, [_i]),
     "tf_gemm_group": (_i, [_vp, _i, _i, _i, _i, _i, _vp, _vp, _i64]),
     "tf_gemm_group_workspace_bytes": (_i64, [_i, _i, _i, _vp]),
     "tf_gemm_workspace_bytes": (_i64, [_i, _i, _i64, _i64, _i64]),
-    "tf_gemm_launch_count": (_i64, []),
-    "tf_gemm_tune": (_i, [_i, _i]),
-    "tf_gemm_debug_flags": (_i, [_i]),
     "tf_attn_fwd": (_i, [_vp, _i, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64,
                          _vp, _vp, _i64, _i64, _f]),
     "tf_attn_bwd": (_i, [_vp, _i, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64,
@@ -61,10 +58,21 @@ SIGNATURES = {
     "tf_softmax_bwd": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64]),
     "tf_cross_entropy_fwd": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _i64, _i64, _vp, _vp, _vp]),
     "tf_cross_entropy_bwd": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _i64, _vp, _i64, _i64]),
-    "tf_colsum": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _vp, _vp, _i64]),
+    "tf_colsum": (_i, [_vp, _i, _i, _i64, _i64, _vp, _i64, _vp, _vp, _i64]),
     "tf_colsum_partial_bytes": (_i64, [_i64, _i64]),
     "tf_relu_mask": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64]),
 }
+
+# include/tritonformer_amd_diag.h: name -> (library, restype, argtypes)
+DIAG_SIGNATURES = {
+    "tf_diag_gemm": ("main", _i, [_vp, _i, _i, _i, _i, _i, _i, _i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64,
+                                  _vp, _i, _vp, _i64]),
+    "tf_diag_gemm_workspace_bytes": ("main", _i64, [_i, _i, _i64, _i64, _i64]),
+    "tf_diag_gemm_launch_count": ("main", _i64, []),
+    "tf_diag_mfma_rate": ("diag", _i, [_vp, _i, _vp, _i, _i, _vp]),
+    "tf_diag_mfma_rate_flops": ("diag", _i64, [_i, _i]),
+}
+
 
 class AdamTensor(ctypes.Structure):
     """tf_adamw_tensor of the C header."""
@@ -78,11 +86,15 @@ class GemmProblem(ctypes.Structure):
                 ("C", _vp), ("ldc", _i64), ("chunk_n", _i64), ("chunk_stride", _i64)]
 
 
+DIAG_LIB_PATH = os.path.join(_HERE, "libtritonformer_amd_diag.so")
+
 _lib = None
+_diag = None
 
 
 def load():
-    """Load the shared library once; raise if it has not been built."""
+    """Load the shared library once; raise if it has not been built, or if it was built
+    from other sources than the ones lying next to it (a stale binary proves nothing)."""
     global _lib
     if _lib is None:
         if not os.path.exists(LIB_PATH):
@@ -95,8 +107,39 @@ def load():
             fn = getattr(lib, name)
             fn.restype = res
             fn.argtypes = args
+        if os.path.isdir(os.path.join(_HERE, "csrc")):
+            from . import _build
+
+            built, here = lib.tf_source_hash().decode(), _build.source_hash()
+            if built != here:
+                raise ImportError(
+                    f"{LIB_PATH} was built from other sources (hash {built or 'none'}) than csrc/ and include/ hold "
+                    f"now ({here}): rebuild it with `python -m tritonformer_amd._build`"
+                )
         _lib = lib
     return _lib
+
+
+class _Diag:
+    """The functions of include/tritonformer_amd_diag.h, wherever they live."""
+
+
+def load_diag():
+    """Diagnostics (benchmark, tests, kernel work); no operator of the package calls this."""
+    global _diag
+    if _diag is None:
+        libs = {"main": load()}
+        if not os.path.exists(DIAG_LIB_PATH):
+            raise ImportError(f"{DIAG_LIB_PATH} is missing: build it with `python -m tritonformer_amd._build`")
+        libs["diag"] = ctypes.CDLL(DIAG_LIB_PATH)
+        d = _Diag()
+        for name, (where, res, args) in DIAG_SIGNATURES.items():
+            fn = getattr(libs[where], name)
+            fn.restype = res
+            fn.argtypes = args
+            setattr(d, name, fn)
+        _diag = d
+    return _diag
 
 
 class TritonformerAmdError(RuntimeError):

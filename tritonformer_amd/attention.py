@@ -5,7 +5,7 @@ from typing import Any, Tuple
 import torch
 from torch.autograd import Function
 
-from ._amp import amp_bwd, amp_fwd
+from ._amp import amp_bwd, amp_fwd, cached_conversion
 from .kernels import (
     cast_pack,
     flash_wrapper_bwd,
@@ -120,7 +120,7 @@ class AttentionBlock(Function):
         hd = d // num_heads
         # the four (d, d) weights side by side in one 16-bit (d, 4d) matrix, one conversion kernel;
         # the GEMMs take its first three column blocks and its last one as strided operands
-        packed = cast_pack([wq, wk, wv, wo], x.dtype)
+        packed = cached_conversion([wq, wk, wv, wo], x.dtype, cast_pack)
         w_qkv, w_o = packed[:, : 3 * d], packed[:, 3 * d:]
         qkv = mm(x, w_qkv).view(b, s, 3, num_heads, hd)
         q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))

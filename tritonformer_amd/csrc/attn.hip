@@ -909,7 +909,10 @@ static int attn_check(int dtype, int64_t B, int64_t nh, int64_t S, int64_t hd, i
   if (dtype != TF_F16 && dtype != TF_BF16) return TF_EDTYPE;
   if (B <= 0 || nh <= 0 || S <= 0) return TF_EINVAL;
   if (hd != 32 && hd != 64 && hd != 128) return TF_ESHAPE;  // as kernels/attention.py:567
-  if (S % 64 != 0) return TF_ESHAPE;                        // as kernels/attention.py:181-183
+  // 64-row blocks for every head_dim (the reference, kernels/attention.py:177-183, uses 32-row
+  // blocks at head_dim 128 and so accepts S % 32 == 0 there: the Python launcher serves those
+  // lengths by continuing the sequence with 32 rows of zeros)
+  if (S % 64 != 0) return TF_ESHAPE;
   if (B * nh * ((S + 127) / 128) > 0x7fffffff || S > (1 << 24)) return TF_EINVAL;
   if (sb % 8 || sh % 8 || ss % 8 || ss < hd) return TF_EALIGN;
   if (osb % 8 || osh % 8 || oss % 8 || oss < hd) return TF_EALIGN;

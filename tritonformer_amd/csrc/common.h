@@ -171,4 +171,10 @@ template <int N, typename F> __device__ __forceinline__ void static_for(F&& f) {
 
 inline int ceil_div(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
 
+// CUs and XCDs of the current device, read from the runtime once per device and kept (the only
+// state this library holds besides the scratch array of the allocation-free entry point).  Falls
+// back to the MI355X figures if the runtime does not answer.
+struct DeviceShape { int cus, xcds; };
+DeviceShape device_shape();
+
 }  // namespace tfa

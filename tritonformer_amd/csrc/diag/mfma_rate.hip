@@ -1,10 +1,11 @@
 // Diagnostic: sustained MFMA rate of the GEMM kernel's instruction stream alone.
-// One workgroup per CU, 8 waves, each issuing the 32 v_mfma_f32_32x32x16 of one 256x256x64
+// `workgroups` workgroups (one per CU is the intended use), 8 waves, each issuing the 32 v_mfma_f32_32x32x16 of one 256x256x64
 // step per loop trip from fixed operand registers -- no memory traffic at all.  The rate
 // depends on the operand VALUES (the chip lowers its clock under the switching activity of
 // random data), which is why the operands are an argument: it is the practical ceiling a
 // GEMM on real data can be compared with.
-#include "rowops.h"
+#include "../rowops.h"
+#include "../../../include/tritonformer_amd_diag.h"
 
 namespace tfa {
 
@@ -48,16 +49,18 @@ __global__ __launch_bounds__(512, 2) void mfma_rate_kernel(const T* __restrict__
 
 using namespace tfa;
 
-extern "C" int64_t tf_probe_mfma_rate_flops(int iters) {
-  return iters > 0 ? (int64_t)iters * 256 * (2ll * 256 * 256 * 64) : 0;
+extern "C" int64_t tf_diag_mfma_rate_flops(int iters, int workgroups) {
+  return iters > 0 && workgroups > 0 ? (int64_t)iters * workgroups * (2ll * 256 * 256 * 64) : 0;
 }
 
-extern "C" int tf_probe_mfma_rate(void* stream, int dtype, const void* operands, int iters, float* sink) {
-  if (!operands || !sink || iters <= 0) return TF_EINVAL;
+extern "C" int tf_diag_mfma_rate(void* stream, int dtype, const void* operands, int iters, int workgroups,
+                                 float* sink) {
+  if (!operands || !sink || iters <= 0 || workgroups <= 0 || workgroups > 65536) return TF_EINVAL;
   if (!aligned16(operands)) return TF_EALIGN;
   hipStream_t st = (hipStream_t)stream;
-  if (dtype == TF_F16) mfma_rate_kernel<f16><<<dim3(256), dim3(512), 0, st>>>((const f16*)operands, iters, sink);
-  else if (dtype == TF_BF16) mfma_rate_kernel<bf16><<<dim3(256), dim3(512), 0, st>>>((const bf16*)operands, iters, sink);
+  const dim3 grid((unsigned)workgroups);
+  if (dtype == TF_F16) mfma_rate_kernel<f16><<<grid, dim3(512), 0, st>>>((const f16*)operands, iters, sink);
+  else if (dtype == TF_BF16) mfma_rate_kernel<bf16><<<grid, dim3(512), 0, st>>>((const bf16*)operands, iters, sink);
   else return TF_EDTYPE;
   TF_CHECK_LAUNCH();
   return TF_OK;

@@ -1,10 +1,17 @@
 // Dense contraction C[M,N] = epilogue(sum_k A(m,k) B(n,k)) on gfx950 MFMA.
 //
-// One workgroup owns a BM x BN tile of C.  Per BK-wide step of the contraction
-// the A and B panels are brought HBM -> registers -> LDS with 16-byte accesses
-// (the next step's loads are in flight while the current step computes, LDS is
-// double buffered, one barrier per step) and consumed by
-// v_mfma_f32_32x32x16_{f16,bf16} with fp32 accumulators.
+// One workgroup owns a BM x BN tile of C (or one slice of its contraction).  Two
+// kernel families share the tiling and the MFMA code:
+//  * gemm_dma_kernel / gemm_dma_group_kernel, the ones a training step runs: per
+//    BK-wide step the A and B panels go HBM -> LDS directly (global_load_lds_dwordx4,
+//    no VGPR round trip) into two LDS stages; the LDS operand reads, the loads of the
+//    next step and the MFMAs are interleaved by hand (bare s_barrier, explicit
+//    s_waitcnt); the result leaves through a wave-private LDS slab so that every
+//    global store covers whole 128-byte lines;
+//  * gemm_kernel, for anything those cannot take (ragged extents, unaligned pointers,
+//    a contraction that is not a multiple of BK): operands staged through registers
+//    with per-element predication, one barrier per step.
+// Both use v_mfma_f32_32x32x16_{f16,bf16} with fp32 accumulators.
 //
 // Either operand may be stored with the contraction dimension contiguous
 // ("K-major": read from LDS with ds_read_b128) or strided ("K-minor": read with
@@ -14,12 +21,11 @@
 // free of bank conflicts.
 //
 // The MFMA is issued as D^T = B_frag x A_frag, so a lane ends up holding four
-// consecutive n for one m: the epilogue (bias, ReLU, rounding) stores 8 bytes
-// per lane and needs no cross-lane traffic.
+// consecutive n for one m: bias, ReLU and rounding need no cross-lane traffic.
 //
-// Workgroup ids are remapped so that each of the 8 XCDs (which receive ids
-// round-robin) works on a compact block of neighbouring tiles and shares the
-// A/B panels through its own L2.
+// Workgroup ids are remapped so that each XCD (which receive ids round-robin)
+// works on a compact block of neighbouring tiles and shares the A/B panels
+// through its own L2.  The number of XCDs and of CUs is read from the device.
 #include <atomic>
 #include <cstdio>
 #include <cstdlib>
@@ -42,7 +48,8 @@ struct GemmParams {
   int relu;
   int splits, k_per_split;
   int tiles_m, tiles_n;
-  int flags;  // bit 0: skip the XCD remap (diagnostic)
+  int flags;  // bit 0: skip the XCD remap (set by the diagnostic entry point only)
+  int xcds;   // XCDs of the device (workgroup ids are dealt to them round-robin)
   int out_f32;  // C holds fp32 instead of T
   const void* mask;  // optional (M, N) activation of type T: C = mask > 0 ? C : 0
   int64_t ldmask;
@@ -138,8 +145,7 @@ struct Panel {
 };
 
 // Round-robin XCD dispatch -> compact per-XCD ranges, then grouped raster.
-__device__ __forceinline__ int remap_xcd(int pid, int n) {
-  constexpr int X = 8;
+__device__ __forceinline__ int remap_xcd(int pid, int n, int X) {
   const int xcd = pid % X, local = pid / X;
   const int q = n / X, r = n % X;
   return xcd * q + (xcd < r ? xcd : r) + local;
@@ -232,7 +238,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_kernel(GemmParams p) {
 
   // ---- which tile / which slice of the contraction -------------------------
   const int tiles = p.tiles_m * p.tiles_n;
-  const int pid = (p.flags & 1) ? (int)blockIdx.x : remap_xcd(blockIdx.x, tiles * p.splits);
+  const int pid = (p.flags & 1) ? (int)blockIdx.x : remap_xcd(blockIdx.x, tiles * p.splits, p.xcds);
   const int split = pid / tiles;
   const int t = pid - split * tiles;
   const int per_group = GROUP_M * p.tiles_n;
@@ -672,7 +678,6 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams& p, const int pid
     }
   }
 
-  if (p.flags & 8) return;
   static_assert(NW * 32 * (WTN * 4 + 16) <= 2 * STAGE, "epilogue staging must fit in the pipeline LDS");
   if (p.splits > 1) {
     // fp32 partial of this contraction slice: a plain (M, N) matrix, written like an fp32 result
@@ -703,7 +708,7 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams& p, const int pid
 
 template <typename T, int BM, int BN, int BK, int WM, int WN, int WPE, bool A_KMAJOR, bool B_KMAJOR>
 __global__ __launch_bounds__(WM* WN * 64, WPE) void gemm_dma_kernel(GemmParams p) {
-  const int pid = (p.flags & 1) ? (int)blockIdx.x : remap_xcd(blockIdx.x, p.tiles_m * p.tiles_n * p.splits);
+  const int pid = (p.flags & 1) ? (int)blockIdx.x : remap_xcd(blockIdx.x, p.tiles_m * p.tiles_n * p.splits, p.xcds);
   gemm_dma_body<T, BM, BN, BK, WM, WN, A_KMAJOR, B_KMAJOR>(p, pid);
 }
 
@@ -718,7 +723,7 @@ struct GemmGroup {
 };
 template <typename T, int BM, int BN, int BK, int WM, int WN, int WPE, bool A_KMAJOR, bool B_KMAJOR>
 __global__ __launch_bounds__(WM* WN * 64, WPE) void gemm_dma_group_kernel(GemmGroup g) {
-  const int pid = remap_xcd(blockIdx.x, g.first[g.count]);
+  const int pid = remap_xcd(blockIdx.x, g.first[g.count], g.p[0].xcds);
   int i = 0;
 #pragma unroll
   for (int k = 1; k < kMaxGroup; ++k)
@@ -822,20 +827,20 @@ static const TileCfg kCfgs[] = {
 };
 constexpr int kNumCfgs = (int)(sizeof(kCfgs) / sizeof(kCfgs[0]));
 
-static int env_int(const char* name, int dflt) {
-  const char* s = getenv(name);
-  return s ? atoi(s) : dflt;
-}
-static int g_force_cfg = env_int("TF_GEMM_CFG", -1);
-static int g_force_splits = env_int("TF_GEMM_SPLITS", 0);
-static int g_flags = env_int("TF_GEMM_FLAGS", 0);
+// What the diagnostic entry point may impose on ONE call (nothing is kept between calls):
+// a tile configuration (index into kCfgs, -1 = chosen by the cost model), a contraction
+// split (0 = chosen), and flag bits -- 1: no XCD remap of the workgroup ids; 64: never cut
+// a product along N.  Every product entry point passes kNoForce.
+struct GemmForce { int cfg, splits, flags; };
+constexpr GemmForce kNoForce = {-1, 0, 0};
 
 // Tile shape, contraction split and the rough cost (microseconds) of running
 // M x N x K with tile configuration `cfg`.  The cost constants are fits to
 // rocprofv3 kernel durations on MI355X: one "round" of workgroups (one per CU)
 // costs a fixed part (launch, cold first loads, result write-out) plus a part
 // per 64-wide contraction step.
-static GemmPlan plan_for(int cfg, int64_t M, int64_t N, int64_t K, double* cost_us, bool allow_split) {
+static GemmPlan plan_for(int cfg, int64_t M, int64_t N, int64_t K, double* cost_us, bool allow_split,
+                         int force_splits = 0) {
   GemmPlan pl;
   pl.cfg = cfg;
   pl.bm = kCfgs[cfg].bm;
@@ -846,7 +851,7 @@ static GemmPlan plan_for(int cfg, int64_t M, int64_t N, int64_t K, double* cost_
   const int64_t tiles = (int64_t)pl.tiles_m * pl.tiles_n;
   const int64_t ksteps = (K + pl.bk - 1) / pl.bk;
   const int wg_per_cu = pl.bm * pl.bn <= 128 * 128 ? 2 : 1;
-  const int64_t slots = 256 * wg_per_cu;
+  const int64_t slots = (int64_t)device_shape().cus * wg_per_cu;
   // Split the contraction only when the tiles alone leave most CUs idle (weight
   // gradients: few output tiles, long contraction); never beyond one full round of
   // workgroups, and every slice keeps at least 16 steps so that the fp32 partial
@@ -858,7 +863,7 @@ static GemmPlan plan_for(int cfg, int64_t M, int64_t N, int64_t K, double* cost_
     if (splits > max_by_k) splits = max_by_k;
     if (splits > 16) splits = 16;
   }
-  if (g_force_splits > 0) splits = g_force_splits;
+  if (force_splits > 0) splits = force_splits;
   if (!allow_split) splits = 1;
   if (splits > ksteps) splits = ksteps > 0 ? ksteps : 1;
   const int64_t steps_per = (ksteps + splits - 1) / splits;
@@ -876,36 +881,14 @@ static GemmPlan plan_for(int cfg, int64_t M, int64_t N, int64_t K, double* cost_
   return pl;
 }
 
-// Diagnostic: TF_GEMM_RULE="M,N,K,cfg[;M,N,K,cfg...]" forces a tile configuration for the given extents only
-// (timing one product of a whole training step under another configuration).
-struct ShapeRule { int64_t m, n, k; int cfg; };
-static int load_rules(ShapeRule* out, int cap) {
-  const char* s = getenv("TF_GEMM_RULE");
-  int n = 0;
-  while (s && *s && n < cap) {
-    long long a, b, c; int cfg, used = 0;
-    if (sscanf(s, "%lld,%lld,%lld,%d%n", &a, &b, &c, &cfg, &used) != 4) break;
-    out[n++] = {a, b, c, cfg};
-    s += used;
-    if (*s == ';') ++s;
-  }
-  return n;
-}
-static ShapeRule g_rules[8];
-static const int g_num_rules = load_rules(g_rules, 8);
-
 static GemmPlan make_plan(int64_t M, int64_t N, int64_t K, bool vec, bool allow_split = true,
-                          double* cost_us = nullptr) {
+                          double* cost_us = nullptr, const GemmForce& force = kNoForce) {
   const bool dma = vec && K % 64 == 0;
   if (cost_us) *cost_us = -1.0;  // stays negative when the configuration is forced
-  for (int i = 0; i < g_num_rules; ++i)
-    if (g_rules[i].m == M && g_rules[i].n == N && g_rules[i].k == K && g_rules[i].cfg >= 0 && g_rules[i].cfg < kNumCfgs &&
-        (!kCfgs[g_rules[i].cfg].dma || dma))
-      return plan_for(g_rules[i].cfg, M, N, K, nullptr, allow_split);
-  if (g_force_cfg >= 0 && g_force_cfg < kNumCfgs) {
-    int cfg = g_force_cfg;
+  if (force.cfg >= 0 && force.cfg < kNumCfgs) {
+    int cfg = force.cfg;
     if (kCfgs[cfg].dma && !dma) cfg = kCfgs[cfg].bm * kCfgs[cfg].bn >= 256 * 256 ? 0 : 1;  // register-staged twin
-    return plan_for(cfg, M, N, K, nullptr, allow_split);
+    return plan_for(cfg, M, N, K, nullptr, allow_split, force.splits);
   }
   // candidates: 256x256 and 256x128 / 128x128 tiles, direct-to-LDS kernels when their
   // preconditions hold, the register-staged twins otherwise
@@ -913,11 +896,11 @@ static GemmPlan make_plan(int64_t M, int64_t N, int64_t K, bool vec, bool allow_
   const int cand_reg[2] = {0, 1};
   const int* cand = dma ? cand_dma : cand_reg;
   const int ncand = dma ? 3 : 2;
-  GemmPlan best = plan_for(cand[0], M, N, K, nullptr, allow_split);
+  GemmPlan best = plan_for(cand[0], M, N, K, nullptr, allow_split, force.splits);
   double best_cost = 1e30;
   for (int i = 0; i < ncand; ++i) {
     double c;
-    const GemmPlan pl = plan_for(cand[i], M, N, K, &c, allow_split);
+    const GemmPlan pl = plan_for(cand[i], M, N, K, &c, allow_split, force.splits);
     if (c < best_cost) { best_cost = c; best = pl; }
   }
   if (cost_us) *cost_us = best_cost;
@@ -1056,21 +1039,13 @@ static int gemm_group_dispatch(hipStream_t st, const GemmGroup& g) {
 
 using namespace tfa;
 
-// Diagnostic: force a tile configuration (index into kCfgs, -1 = automatic) and
-// a contraction split (0 = automatic) for every later tf_gemm call.
-extern "C" int tf_gemm_tune(int cfg, int splits) {
-  if (cfg >= kNumCfgs) return TF_EINVAL;
-  g_force_cfg = cfg;
-  g_force_splits = splits;
-  return TF_OK;
-}
+extern "C" int64_t tf_diag_gemm_launch_count(void) { return g_gemm_launches.load(std::memory_order_relaxed); }
 
-extern "C" int64_t tf_gemm_launch_count(void) { return g_gemm_launches.load(std::memory_order_relaxed); }
-
-// Diagnostic: bit 0 skips the XCD remap, bit 3 skips the epilogue (timing only, wrong results).
-extern "C" int tf_gemm_debug_flags(int flags) {
-  g_flags = flags;
-  return TF_OK;
+// Tile columns (of 256x256 tiles) per whole number of rounds of workgroups, one per CU.
+static int64_t round_unit(int64_t tiles_m, int64_t cus) {
+  int64_t a = tiles_m, b = cus;
+  while (b) { const int64_t t = a % b; a = b; b = t; }
+  return cus / a;
 }
 
 // A product whose 256x256 tiles fill a whole number of rounds of workgroups plus a small
@@ -1078,20 +1053,19 @@ extern "C" int tf_gemm_debug_flags(int flags) {
 // that runs as a split contraction on the otherwise idle CUs instead of a nearly empty last
 // round (LM-head weight gradient: 4 x 197 tiles = 3 rounds + 20 tiles).  Returns the number
 // of tail columns, 0 for no cut.
-static int64_t tail_columns(int64_t M, int64_t N, int64_t K, bool vec, bool allow_split) {
-  if (!allow_split || g_force_cfg >= 0 || g_force_splits > 0 || K < 32 * 64 || (g_flags & 64)) return 0;
+static int64_t tail_columns(int64_t M, int64_t N, int64_t K, bool vec, bool allow_split, const GemmForce& force) {
+  if (!allow_split || force.cfg >= 0 || force.splits > 0 || K < 32 * 64 || (force.flags & 64)) return 0;
+  const int64_t cus = device_shape().cus;
   double uncut;
   const GemmPlan pl = make_plan(M, N, K, vec, allow_split, &uncut);
   const int64_t tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
-  int64_t a = tiles_m, b = 256;
-  while (b) { const int64_t t = a % b; a = b; b = t; }
-  const int64_t unit = 256 / a;  // tile columns per whole number of rounds
+  const int64_t unit = round_unit(tiles_m, cus);
   const int64_t tn1 = (tiles_n / unit) * unit;
   if (tn1 <= 0 || tn1 * 256 >= N) return 0;
   if (pl.cfg == 2 && pl.splits == 1) {
     const int64_t tiles = tiles_m * tiles_n;
-    const int64_t rem = tiles % 256;
-    if (tiles > 256 && rem != 0 && rem <= 64) return N - tn1 * 256;
+    const int64_t rem = tiles % cus;
+    if (tiles > cus && rem != 0 && rem <= cus / 4) return N - tn1 * 256;
   }
   return 0;
 }
@@ -1101,16 +1075,15 @@ static int64_t tail_columns(int64_t M, int64_t N, int64_t K, bool vec, bool allo
 // together are cheaper than the best single launch (q/k/v projection 8192 x 3072 x 1024: one
 // round of 256x256 tiles + 1024 columns of 128x128 tiles, 0.2 ms per training step less than
 // three rounds of 128x128 tiles).
-static int64_t round_cut_columns(int64_t M, int64_t N, int64_t K, bool vec, bool allow_split) {
-  if (!allow_split || g_force_cfg >= 0 || g_force_splits > 0 || !(vec && K % 64 == 0) || (g_flags & 64)) return 0;
+static int64_t round_cut_columns(int64_t M, int64_t N, int64_t K, bool vec, bool allow_split, const GemmForce& force) {
+  if (!allow_split || force.cfg >= 0 || force.splits > 0 || !(vec && K % 64 == 0) || (force.flags & 64)) return 0;
+  const int64_t cus = device_shape().cus;
   double uncut, whole, rest;
   (void)make_plan(M, N, K, vec, allow_split, &uncut);
   if (uncut < 0) return 0;
   const int64_t tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
-  if (tiles_m * tiles_n <= 256) return 0;
-  int64_t a = tiles_m, b = 256;
-  while (b) { const int64_t t = a % b; a = b; b = t; }
-  const int64_t unit = 256 / a;
+  if (tiles_m * tiles_n <= cus) return 0;
+  const int64_t unit = round_unit(tiles_m, cus);
   const int64_t tn1 = (tiles_n / unit) * unit;
   if (tn1 <= 0 || tn1 * 256 >= N) return 0;
   (void)plan_for(2, M, tn1 * 256, K, &whole, false);
@@ -1132,8 +1105,8 @@ extern "C" int64_t tf_gemm_workspace_bytes(int layout_a, int layout_b, int64_t M
   int64_t need = 0;
   for (int vec = 0; vec < 2; ++vec) {
     int64_t n = single_need(M, N, K, vec != 0);
-    int64_t tail = tail_columns(M, N, K, vec != 0, true);
-    if (tail == 0) tail = round_cut_columns(M, N, K, vec != 0, true);
+    int64_t tail = tail_columns(M, N, K, vec != 0, true, kNoForce);
+    if (tail == 0) tail = round_cut_columns(M, N, K, vec != 0, true, kNoForce);
     if (tail > 0) {
       const int64_t n1 = single_need(M, N - tail, K, vec != 0), n2 = single_need(M, tail, K, vec != 0);
       if (n1 > n) n = n1;
@@ -1163,7 +1136,7 @@ static int gemm_entry(void* stream, int dtype, int out_dtype, int layout_a, int 
                       int64_t K, const void* A, int64_t lda, const void* B, int64_t ldb, void* C, int64_t ldc,
                       int64_t chunk_n, int64_t chunk_stride, const void* bias, int relu, const void* mask_act,
                       int64_t ld_mask, void* workspace, int64_t workspace_bytes, void* sign_out, const void* sign_in,
-                      int64_t ld_sign) {
+                      int64_t ld_sign, const GemmForce& force = kNoForce) {
   if (!A || !B || !C) return TF_EINVAL;
   const bool signs = sign_out || sign_in;
   if (signs) {
@@ -1192,23 +1165,22 @@ static int gemm_entry(void* stream, int dtype, int out_dtype, int layout_a, int 
                    b_contig % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 && N % 8 == 0 && ldc % 8 == 0 &&
                    (!mask_act || (aligned16(mask_act) && ld_mask % 8 == 0));
   if (chunk_n == N && !signs) {
-    int64_t tail = tail_columns(M, N, K, vec, mask_act == nullptr);
-    if (tail == 0) tail = round_cut_columns(M, N, K, vec, mask_act == nullptr);
+    int64_t tail = tail_columns(M, N, K, vec, mask_act == nullptr, force);
+    if (tail == 0) tail = round_cut_columns(M, N, K, vec, mask_act == nullptr, force);
     if (tail > 0) {  // whole rounds first, then the narrow remainder as a split contraction
       const int64_t n1 = N - tail;
       const int64_t osz = out_dtype == TF_F32 ? 4 : 2;
       const char* b2 = (const char*)B + (layout_b == TF_OP_KMAJOR ? n1 * ldb : n1) * 2;
       const void* bias2 = bias ? (const char*)bias + n1 * 2 : nullptr;
       const void* mask2 = mask_act ? (const char*)mask_act + n1 * 2 : nullptr;
-      const int rc = tf_gemm_out_chunked(stream, dtype, out_dtype, layout_a, layout_b, M, n1, K, A, lda, B, ldb, C, ldc,
-                                         0, 0, bias, relu, mask_act, ld_mask, workspace, workspace_bytes);
+      const int rc = gemm_entry(stream, dtype, out_dtype, layout_a, layout_b, M, n1, K, A, lda, B, ldb, C, ldc, 0, 0, bias,
+                                relu, mask_act, ld_mask, workspace, workspace_bytes, nullptr, nullptr, 0, force);
       if (rc != TF_OK) return rc;
-      return tf_gemm_out_chunked(stream, dtype, out_dtype, layout_a, layout_b, M, tail, K, A, lda, b2, ldb,
-                                 (char*)C + n1 * osz, ldc, 0, 0, bias2, relu, mask2, ld_mask, workspace,
-                                 workspace_bytes);
+      return gemm_entry(stream, dtype, out_dtype, layout_a, layout_b, M, tail, K, A, lda, b2, ldb, (char*)C + n1 * osz,
+                        ldc, 0, 0, bias2, relu, mask2, ld_mask, workspace, workspace_bytes, nullptr, nullptr, 0, force);
     }
   }
-  const GemmPlan pl = make_plan(M, N, K, vec, mask_act == nullptr && !signs);
+  const GemmPlan pl = make_plan(M, N, K, vec, mask_act == nullptr && !signs, nullptr, force);
   // the sign bits exist in the write-out of the direct-to-LDS kernels only
   if (signs && !(kCfgs[pl.cfg].dma && vec && K % pl.bk == 0 && pl.splits == 1)) return TF_EINVAL;
   const int64_t need = pl.splits > 1 ? (int64_t)pl.splits * M * N * (int64_t)sizeof(float) : 0;
@@ -1223,7 +1195,8 @@ static int gemm_entry(void* stream, int dtype, int out_dtype, int layout_a, int 
   p.relu = relu ? 1 : 0;
   p.splits = pl.splits; p.k_per_split = pl.k_per_split;
   p.tiles_m = pl.tiles_m; p.tiles_n = pl.tiles_n;
-  p.flags = g_flags;
+  p.flags = force.flags;
+  p.xcds = device_shape().xcds;
   p.out_f32 = out_dtype == TF_F32 ? 1 : 0;
   p.mask = mask_act;
   p.ldmask = ld_mask;
@@ -1255,6 +1228,30 @@ extern "C" int tf_gemm_relu_bits(void* stream, int dtype, int out_dtype, int lay
                     bits_out ? 1 : 0, nullptr, 0, nullptr, 0, bits_out, bits_in, ld_bits);
 }
 
+// Diagnostic twin of tf_gemm_out_chunked: the same call with a tile configuration, a contraction
+// split and flag bits imposed on THIS call only (no state is kept).
+extern "C" int tf_diag_gemm(void* stream, int cfg, int splits, int flags, int dtype, int out_dtype, int layout_a,
+                            int layout_b, int64_t M, int64_t N, int64_t K, const void* A, int64_t lda, const void* B,
+                            int64_t ldb, void* C, int64_t ldc, const void* bias, int relu, void* workspace,
+                            int64_t workspace_bytes) {
+  if (cfg >= kNumCfgs || splits < 0 || (flags & ~(1 | 64))) return TF_EINVAL;
+  const GemmForce force = {cfg < 0 ? -1 : cfg, splits, flags};
+  return gemm_entry(stream, dtype, out_dtype, layout_a, layout_b, M, N, K, A, lda, B, ldb, C, ldc, 0, 0, bias, relu,
+                    nullptr, 0, workspace, workspace_bytes, nullptr, nullptr, 0, force);
+}
+extern "C" int64_t tf_diag_gemm_workspace_bytes(int cfg, int splits, int64_t M, int64_t N, int64_t K) {
+  if (M <= 0 || N <= 0 || K <= 0 || cfg >= kNumCfgs) return 0;
+  if (cfg < 0 && splits <= 0) return tf_gemm_workspace_bytes(0, 0, M, N, K);
+  const GemmForce force = {cfg < 0 ? -1 : cfg, splits, 0};
+  int64_t need = 0;
+  for (int vec = 0; vec < 2; ++vec) {
+    const GemmPlan pl = make_plan(M, N, K, vec != 0, true, nullptr, force);
+    const int64_t n = pl.splits > 1 ? (int64_t)pl.splits * M * N * (int64_t)sizeof(float) : 0;
+    if (n > need) need = n;
+  }
+  return need;
+}
+
 // ---- grouped products -------------------------------------------------------
 namespace {
 
@@ -1279,8 +1276,8 @@ bool group_problem_fast(const tf_gemm_problem& q) {
 
 GroupPlan plan_group(int la, int lb, int count, const tf_gemm_problem* pr) {
   GroupPlan gp = {false, 1, 0};
-  bool fast = count >= 2 && count <= kMaxGroup && la == TF_OP_KMINOR && lb == TF_OP_KMINOR && g_force_cfg < 0 &&
-              g_force_splits <= 0;
+  bool fast = count >= 2 && count <= kMaxGroup && la == TF_OP_KMINOR && lb == TF_OP_KMINOR;
+  const int64_t cus = device_shape().cus;
   int64_t tiles = 0, min_ksteps = INT64_MAX;
   for (int i = 0; i < count && fast; ++i) {
     fast = group_problem_ok(pr[i]) && group_problem_fast(pr[i]);
@@ -1293,8 +1290,8 @@ GroupPlan plan_group(int la, int lb, int count, const tf_gemm_problem* pr) {
     // same rule as for a single product: split only when the tiles alone leave most CUs idle,
     // never beyond one round of workgroups, slices of at least 16 steps
     int64_t splits = 1;
-    if (tiles <= 128) {
-      splits = 256 / tiles;
+    if (tiles <= cus / 2) {
+      splits = cus / tiles;
       const int64_t max_by_k = min_ksteps / 16 > 0 ? min_ksteps / 16 : 1;
       if (splits > max_by_k) splits = max_by_k;
       if (splits > 16) splits = 16;
@@ -1355,7 +1352,8 @@ extern "C" int tf_gemm_group(void* stream, int dtype, int out_dtype, int layout_
     const int64_t steps_per = (ksteps + gp.splits - 1) / gp.splits;
     p.k_per_split = (int)(steps_per * 64);
     p.splits = (int)((ksteps + steps_per - 1) / steps_per);
-    p.flags = g_flags;
+    p.flags = 0;
+    p.xcds = device_shape().xcds;
     p.out_f32 = out_dtype == TF_F32 ? 1 : 0;
     p.mask = nullptr; p.ldmask = 0;
     p.sign_out = nullptr; p.sign_in = nullptr; p.ldsign = 0;

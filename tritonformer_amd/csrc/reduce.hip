@@ -116,7 +116,7 @@ __global__ __launch_bounds__(256) void relu_mask_kernel(int64_t rows, int cols, 
 
 template <typename T>
 static int colsum_launch(hipStream_t st, int64_t rows, int64_t cols, const void* x, int64_t ldx, void* out,
-                         float* partial) {
+                         bool out_f32, float* partial) {
   const int groups = colsum_groups(rows, cols);
   const int rpg = (int)((rows + groups - 1) / groups);
   const dim3 grid((unsigned)ceil_div(cols, kCsColsPerBlock), (unsigned)groups), block(256);
@@ -125,7 +125,8 @@ static int colsum_launch(hipStream_t st, int64_t rows, int64_t cols, const void*
   else
     colsum_partial<T, false><<<grid, block, 0, st>>>(rows, (int)cols, (const T*)x, ldx, partial, rpg);
   TF_CHECK_LAUNCH();
-  colsum_final<T><<<dim3(ceil_div(cols, 32)), block, 0, st>>>(groups, (int)cols, partial, (T*)out);
+  if (out_f32) colsum_final<float><<<dim3(ceil_div(cols, 32)), block, 0, st>>>(groups, (int)cols, partial, (float*)out);
+  else colsum_final<T><<<dim3(ceil_div(cols, 32)), block, 0, st>>>(groups, (int)cols, partial, (T*)out);
   TF_CHECK_LAUNCH();
   return TF_OK;
 }
@@ -200,15 +201,16 @@ extern "C" int64_t tf_colsum_partial_bytes(int64_t rows, int64_t cols) {
   return (int64_t)colsum_groups(rows, cols) * cols * (int64_t)sizeof(float);
 }
 
-extern "C" int tf_colsum(void* stream, int dtype, int64_t rows, int64_t cols, const void* x, int64_t ldx, void* out,
-                         float* partial, int64_t partial_bytes) {
+extern "C" int tf_colsum(void* stream, int dtype, int out_dtype, int64_t rows, int64_t cols, const void* x,
+                         int64_t ldx, void* out, float* partial, int64_t partial_bytes) {
   if (!x || !out) return TF_EINVAL;
   if (rows <= 0 || cols <= 0 || cols > (1 << 30) || ldx < cols) return TF_EINVAL;
+  if (dtype != TF_F16 && dtype != TF_BF16) return TF_EDTYPE;
+  if (out_dtype != dtype && out_dtype != TF_F32) return TF_EDTYPE;
   if (!partial || partial_bytes < tf_colsum_partial_bytes(rows, cols)) return TF_EWORKSPACE;
   hipStream_t st = (hipStream_t)stream;
-  if (dtype == TF_F16) return colsum_launch<f16>(st, rows, cols, x, ldx, out, partial);
-  if (dtype == TF_BF16) return colsum_launch<bf16>(st, rows, cols, x, ldx, out, partial);
-  return TF_EDTYPE;
+  if (dtype == TF_F16) return colsum_launch<f16>(st, rows, cols, x, ldx, out, out_dtype == TF_F32, partial);
+  return colsum_launch<bf16>(st, rows, cols, x, ldx, out, out_dtype == TF_F32, partial);
 }
 
 extern "C" int tf_relu_mask(void* stream, int dtype, int64_t rows, int64_t cols, const void* grad, int64_t ldg,

@@ -127,8 +127,11 @@ def gemm_relu_bits(a, b, bias=None):
     return out, None
 
 
-def mm_masked_bits(a, b, bits):
-    """``(a @ b) * mask`` with the mask given as the sign bits of gemm_relu_bits."""
+def mm_masked_bits(a, b, bits, act=None):
+    """``(a @ b) * mask`` with the mask given as the sign bits of gemm_relu_bits.  The kernel that
+    reads the bits has preconditions of its own (whole 64-wide contraction steps, aligned
+    operands) which this product may miss although the one that wrote the bits met them; ``act``,
+    the activation the bits were taken from, then serves as the mask (``mm(..., mask_act=act)``)."""
     _check_linear(a, b, None)
     a2, m, k = _rows2d(a)
     n = b.shape[1]
@@ -137,7 +140,10 @@ def mm_masked_bits(a, b, bits):
     require_cuda(bits)
     b, lb, ldb = _operand_b(b, n, k)
     out = torch.empty(a.shape[:-1] + (n,), dtype=a.dtype, device=a.device)
-    check(_gemm_bits(a.dtype, lb, m, n, k, a2, b, ldb, out, None, None, bits))
+    rc = _gemm_bits(a.dtype, lb, m, n, k, a2, b, ldb, out, None, None, bits)
+    if rc != 0 and act is not None:
+        return gemm(a, b, None, False, act)
+    check(rc)
     return out
 
 
@@ -269,17 +275,18 @@ def embedding_bwd(grad_out, ids, tok_shape, pos_shape, param_dtype):
     return d_tok, d_pos
 
 
-def unbroadcast_leading(x):
+def unbroadcast_leading(x, out_dtype=None):
     """Sum over every dimension but the last, fp32 accumulation -> (cols,)
-    (reference kernels/reductions.py:97-122)."""
+    (reference kernels/reductions.py:97-122).  ``out_dtype=torch.float32`` stores the fp32 sums
+    unrounded (gradient of an fp32 master bias)."""
     require_cuda(x)
     lib = load()
     x2, rows, cols = _rows2d(x)
-    out = torch.empty((cols,), dtype=x.dtype, device=x.device)
+    out = torch.empty((cols,), dtype=out_dtype or x.dtype, device=x.device)
     pb = lib.tf_colsum_partial_bytes(rows, cols)
     part = torch.empty(pb, dtype=torch.uint8, device=x.device)
-    check(lib.tf_colsum(stream_ptr(), dtype_code(x.dtype), rows, cols, x2.data_ptr(), cols, out.data_ptr(),
-                        part.data_ptr(), pb))
+    check(lib.tf_colsum(stream_ptr(), dtype_code(x.dtype), dtype_code(out.dtype), rows, cols, x2.data_ptr(), cols,
+                        out.data_ptr(), part.data_ptr(), pb))
     return out
 
 
@@ -314,8 +321,9 @@ def _check_attn(q, k, v, bias):
     b, nh, s, hd = q.shape
     if hd not in (32, 64, 128):
         raise ValueError("Only head_dims of [32,64,128] are supported.")
-    if s % 64 != 0:
-        raise ValueError("Sequence length must be a multiple of the 64-row block size")
+    # kernels/attention.py:177-183 of the reference: 64-row blocks, 32-row blocks at head_dim 128
+    if s % (32 if hd == 128 else 64) != 0:
+        raise ValueError("Sequence length must be a multiple of the block size (64; 32 at head_dim 128)")
     if not (q.dtype == k.dtype == v.dtype) or q.dtype not in (torch.float16, torch.bfloat16):
         raise TypeError("q, k, v must share one 16-bit dtype")
     require_cuda(q, k, v, bias)
@@ -349,16 +357,46 @@ def _strided_ok(t):
     return t.stride(-1) == 1 and all(st % 8 == 0 for st in t.stride()[:-1]) and t.data_ptr() % 16 == 0
 
 
+def _pad_seq(t, pad):
+    """(B, nh, S, hd) -> contiguous (B, nh, S + pad, hd), zeros below."""
+    b, nh, s, hd = t.shape
+    out = torch.zeros((b, nh, s + pad, hd), dtype=t.dtype, device=t.device)
+    out[:, :, :s].copy_(t)
+    return out
+
+
+def _pad_bias(bias, need):
+    """A dense (nh, S', S') bias grown to S' >= need with zeros (what the extra rows and columns
+    hold never reaches a real query: their keys lie above its diagonal); slopes pass through."""
+    if bias is None or bias.ndim == 1 or bias.shape[1] >= need:
+        return bias
+    nh, sb, _ = bias.shape
+    out = torch.zeros((nh, need, need), dtype=bias.dtype, device=bias.device)
+    out[:, :sb, :sb].copy_(bias)
+    return out
+
+
 def flash_wrapper_fwd(q, k, v, bias=None, out=None):
     """Causal attention forward -> (out, lse).  ``bias``: None, a dense (nh, S', S') matrix, or
     the (nh,) float16 ALiBi slopes (the bias -slope_h * (i - j) is then computed in the kernel
     with the roundings of the reference's dense matrix).  ``out`` has q's strides unless a
     (B, nh, S, hd) view is passed in; ``lse`` is (B, nh, S) fp32 in the log2
     domain (the reference keeps fp16 m and l, kernels/attention.py:171-217 and
-    kernels/biased_attention.py:188-245)."""
+    kernels/biased_attention.py:188-245); (B, nh, S + 32) when S is not a multiple of 64."""
     _check_attn(q, k, v, bias)
-    q, k, v = _attn_layout(q, k, v)
     b, nh, s, hd = q.shape
+    if s % 64:
+        # head_dim 128 with S = 32 (mod 64), which the reference serves with 32-row blocks: the
+        # kernels work on 64-row blocks, so the sequence is continued by 32 rows of zeros.  Under
+        # the causal mask no real query sees an added key, and the added queries are dropped.  The
+        # log-sum-exp comes back for all S + 32 rows: the backward needs those of the added rows.
+        pad = 64 - s % 64
+        o_p, lse = flash_wrapper_fwd(_pad_seq(q, pad), _pad_seq(k, pad), _pad_seq(v, pad), _pad_bias(bias, s + pad))
+        if out is None:
+            out = torch.empty_strided(q.shape, q.stride(), dtype=q.dtype, device=q.device)
+        out.copy_(o_p[:, :, :s])
+        return out, lse
+    q, k, v = _attn_layout(q, k, v)
     if out is None:
         out = torch.empty_strided(q.shape, q.stride(), dtype=q.dtype, device=q.device)
     elif out.shape != q.shape or out.dtype != q.dtype or not _strided_ok(out):
@@ -383,6 +421,20 @@ def flash_wrapper_bwd(grad_out, out, q, k, v, lse, bias=None, grads=None):
     into the three (B, nh, S, hd) views given as ``grads``); reference
     kernels/attention.py:550-607, kernels/biased_attention.py:598-660."""
     _check_attn(q, k, v, bias)
+    if q.shape[2] % 64:
+        # the zero-continued sequence of flash_wrapper_fwd: added rows carry zero output gradient,
+        # so they add nothing to dk, dv; their dq rows are dropped
+        s = q.shape[2]
+        pad = 64 - s % 64
+        if lse.shape[-1] != s + pad:
+            raise ValueError("lse must be the one flash_wrapper_fwd returned for this sequence")
+        got = flash_wrapper_bwd(_pad_seq(grad_out, pad), _pad_seq(out, pad), _pad_seq(q, pad), _pad_seq(k, pad),
+                                _pad_seq(v, pad), lse, _pad_bias(bias, s + pad))
+        if grads is None:
+            grads = tuple(torch.empty_strided(q.shape, q.stride(), dtype=q.dtype, device=q.device) for _ in range(3))
+        for dst, src in zip(grads, got):
+            dst.copy_(src[:, :, :s])
+        return grads
     q, k, v = _attn_layout(q, k, v)
     if not _strided_ok(out):
         out = out.contiguous()

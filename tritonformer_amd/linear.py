@@ -3,7 +3,7 @@ the reference's tritonformer/linear.py.  Weight layout is (in, out): y = x @ W."
 import torch
 from torch.autograd import Function
 
-from ._amp import amp_bwd, amp_fwd
+from ._amp import amp_bwd, amp_fwd, cached_conversion
 from .kernels import (cast_pack, gemm, gemm_relu_bits, mask_grad, mm, mm_dw, mm_dw_group, mm_masked_bits,
                       unbroadcast_leading)
 
@@ -14,6 +14,12 @@ GROUP_DW = True
 RELU_BITS = True
 # True: fp32 master weights of one block are converted to 16 bits by one kernel launch, not one each
 PACK_CASTS = True
+
+
+def _bias_grad(ctx, grad, index):
+    """Column sums of ``grad`` as the gradient of the bias passed at argument ``index``: fp32 sums
+    stored unrounded for an fp32 master bias (as the weight gradients are), else in 16 bits."""
+    return unbroadcast_leading(grad, torch.float32 if ctx.arg_dtypes[index] == torch.float32 else None)
 
 
 def _grads(ctx, grad_output, inputs, weights):
@@ -61,7 +67,7 @@ class LinearBias(Function):
     def backward(ctx, grad_output):
         inputs, weights = ctx.saved_tensors
         grad_input, grad_weights = _grads(ctx, grad_output, inputs, weights)
-        grad_bias = unbroadcast_leading(grad_output) if ctx.needs_input_grad[2] else None
+        grad_bias = _bias_grad(ctx, grad_output, 2) if ctx.needs_input_grad[2] else None
         return grad_input, grad_weights, grad_bias
 
 
@@ -99,7 +105,7 @@ class LinearBiasReLU(Function):
         inputs, weights, out_w_act = ctx.saved_tensors
         grad_output = mask_grad(grad_output, out_w_act)
         grad_input, grad_weights = _grads(ctx, grad_output, inputs, weights)
-        grad_bias = unbroadcast_leading(grad_output) if ctx.needs_input_grad[2] else None
+        grad_bias = _bias_grad(ctx, grad_output, 2) if ctx.needs_input_grad[2] else None
         return grad_input, grad_weights, grad_bias
 
 
@@ -120,7 +126,8 @@ class MLPReLU(Function):
             # they are stored alike (two matrices of d*f elements each seen as two rows)
             if (PACK_CASTS and w1.dtype == w2.dtype == torch.float32 and w1.numel() == w2.numel()
                     and w1.is_contiguous() and w2.is_contiguous() and w1.numel() % 8 == 0):
-                both = cast_pack([w1.view(1, -1), w2.view(1, -1)], input.dtype)
+                both = cached_conversion([w1, w2], input.dtype,
+                                         lambda ws, dt: cast_pack([ws[0].view(1, -1), ws[1].view(1, -1)], dt))
                 w1, w2 = both[0, : w1.numel()].view(w1.shape), both[0, w1.numel():].view(w2.shape)
             else:
                 w1, w2 = w1.to(input.dtype), w2.to(input.dtype)
@@ -140,10 +147,12 @@ class MLPReLU(Function):
         input, w1, w2, hidden = ctx.saved_tensors
         f32 = torch.float32
         if ctx.relu_bits is not None:
-            grad_hidden = mm_masked_bits(grad_output, w2.T, ctx.relu_bits)  # (dY W2^T) * (hidden > 0)
+            # (dY W2^T) * (hidden > 0); `hidden` itself is the mask where this product (contraction
+            # over d_out) misses the preconditions that the forward one (over d_in) met
+            grad_hidden = mm_masked_bits(grad_output, w2.T, ctx.relu_bits, act=hidden)
         else:
             grad_hidden = mm(grad_output, w2.T, mask_act=hidden)
-        grad_b2 = unbroadcast_leading(grad_output) if ctx.has_bias[1] else None
+        grad_b2 = _bias_grad(ctx, grad_output, 4) if ctx.has_bias[1] else None
         # the weight gradients first, the input gradient last: what the next kernel of the backward
         # pass reads is then what was written last (0.1 ms per step of the 410M model)
         if GROUP_DW and ctx.arg_dtypes[1] == ctx.arg_dtypes[3]:
@@ -153,7 +162,7 @@ class MLPReLU(Function):
         else:
             grad_w2 = mm_dw(hidden, grad_output, out_dtype=f32 if ctx.arg_dtypes[3] == f32 else None)
             grad_w1 = mm_dw(input, grad_hidden, out_dtype=f32 if ctx.arg_dtypes[1] == f32 else None)
-        grad_b1 = unbroadcast_leading(grad_hidden) if ctx.has_bias[0] else None
+        grad_b1 = _bias_grad(ctx, grad_hidden, 2) if ctx.has_bias[0] else None
         grad_input = mm(grad_hidden, w1.T) if ctx.needs_input_grad[0] else None
         return grad_input, grad_w1, grad_b1, grad_w2, grad_b2
 
@@ -170,7 +179,7 @@ class PackedLinearNoBias(Function):
     @staticmethod
     @amp_fwd(keep=(1, 2, 3, 4))
     def forward(ctx, input, *weights):
-        packed = cast_pack(weights, input.dtype)
+        packed = cached_conversion(list(weights), input.dtype, cast_pack)
         ctx.save_for_backward(input, packed)
         ctx.count = len(weights)
         ctx.weight_dtype = weights[0].dtype

@@ -65,4 +65,8 @@ class AdamW(torch.optim.Optimizer):
                 check(lib.tf_adamw_step(stream_ptr(), dtype_code(self.shadow_dtype or torch.float16), len(items),
                                         ctypes.cast(arr, ctypes.c_void_p), group["lr"], group["betas"][0],
                                         group["betas"][1], group["eps"], group["weight_decay"], step))
+                # the kernel wrote through raw pointers: tell autograd (and anything keyed on the
+                # version counter, like the cache of 16-bit weight copies) that the values changed
+                for p, _, _ in items:
+                    torch.autograd.graph.increment_version(p)
         return loss
