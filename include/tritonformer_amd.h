@@ -332,6 +332,18 @@ int tf_colsum(void* stream, int dtype, int out_dtype, int64_t rows, int64_t cols
               float* partial, int64_t partial_bytes);
 int64_t tf_colsum_partial_bytes(int64_t rows, int64_t cols);
 
+/* tf_colsum for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc): same kernels and results, bit for bit, with the
+ * first-stage partial sums in a fixed 4 MiB array inside the library instead of a `partial`
+ * buffer.  No counterpart in the reference.  The call allocates and frees nothing.
+ * Limit: problems whose tf_colsum_partial_bytes(rows, cols) exceeds
+ * tf_colsum_noalloc_max_partial_bytes() (4 MiB; the partial sums of a problem take about 2 MiB
+ * whatever its shape, more only beyond a million columns) are refused with TF_EWORKSPACE.  Every call on one GPU uses that GPU's one array: calls that overlap in time on
+ * one GPU (two streams, two threads) race; calls on one stream are ordered and safe. */
+int tf_colsum_noalloc(void* stream, int dtype, int out_dtype, int64_t rows, int64_t cols,
+                      const void* x, int64_t ldx, void* out);
+int64_t tf_colsum_noalloc_max_partial_bytes(void);
+
 /* out = where(act > 0, grad, 0), out of place.
  * Replaces mask_grad (kernels/activation.py:27-44), which works in place. */
 int tf_relu_mask(void* stream, int dtype, int64_t rows, int64_t cols,

@@ -60,6 +60,8 @@ SIGNATURES = {
     "tf_cross_entropy_bwd": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _i64, _vp, _i64, _i64]),
     "tf_colsum": (_i, [_vp, _i, _i, _i64, _i64, _vp, _i64, _vp, _vp, _i64]),
     "tf_colsum_partial_bytes": (_i64, [_i64, _i64]),
+    "tf_colsum_noalloc": (_i, [_vp, _i, _i, _i64, _i64, _vp, _i64, _vp]),
+    "tf_colsum_noalloc_max_partial_bytes": (_i64, []),
     "tf_relu_mask": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64]),
 }
 

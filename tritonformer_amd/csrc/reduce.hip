@@ -1,8 +1,16 @@
 // Column sums (bias gradient) and the ReLU gradient mask for gfx950; both are
 // HBM-bound streaming kernels with 16-byte accesses.
+#include <atomic>
 #include "rowops.h"
 
 namespace tfa {
+
+// Scratch of the allocation-free column sum (tf_colsum_noalloc): the first-stage partial sums live
+// here instead of in a buffer the caller brings.  One copy per GPU the library runs on, held until
+// the process ends.  In host code the array's name is only a handle for hipGetSymbolAddress; the
+// device address it yields is what kernels and copies are given.
+constexpr int64_t kNoAllocScratchBytes = 4 << 20;
+static __device__ __align__(256) float scratch[kNoAllocScratchBytes / sizeof(float)];
 
 constexpr int kCsColsPerBlock = 256;  // 32 lanes x 8 elements
 constexpr int kCsSlices = 8;          // row slices per workgroup
@@ -209,6 +217,44 @@ extern "C" int tf_colsum(void* stream, int dtype, int out_dtype, int64_t rows, i
   if (out_dtype != dtype && out_dtype != TF_F32) return TF_EDTYPE;
   if (!partial || partial_bytes < tf_colsum_partial_bytes(rows, cols)) return TF_EWORKSPACE;
   hipStream_t st = (hipStream_t)stream;
+  if (dtype == TF_F16) return colsum_launch<f16>(st, rows, cols, x, ldx, out, out_dtype == TF_F32, partial);
+  return colsum_launch<bf16>(st, rows, cols, x, ldx, out, out_dtype == TF_F32, partial);
+}
+
+// Device address of `scratch` on the current device, looked up once per device (with that device
+// current) and kept.  Returns null if the runtime refuses.
+static float* noalloc_scratch() {
+  constexpr int kMaxDevices = 64;
+  static std::atomic<float*> ptrs[kMaxDevices];
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  float* p = ptrs[dev].load(std::memory_order_acquire);
+  if (!p) {
+    void* addr = nullptr;
+    if (hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch)) != hipSuccess || !addr) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    p = static_cast<float*>(addr);
+    ptrs[dev].store(p, std::memory_order_release);  // every thread finds the same address
+  }
+  return p;
+}
+
+extern "C" int64_t tf_colsum_noalloc_max_partial_bytes(void) { return kNoAllocScratchBytes; }
+
+extern "C" int tf_colsum_noalloc(void* stream, int dtype, int out_dtype, int64_t rows, int64_t cols, const void* x,
+                                 int64_t ldx, void* out) {
+  if (!x || !out) return TF_EINVAL;
+  if (rows <= 0 || cols <= 0 || cols > (1 << 30) || ldx < cols) return TF_EINVAL;
+  if (dtype != TF_F16 && dtype != TF_BF16) return TF_EDTYPE;
+  if (out_dtype != dtype && out_dtype != TF_F32) return TF_EDTYPE;
+  if (tf_colsum_partial_bytes(rows, cols) > kNoAllocScratchBytes) return TF_EWORKSPACE;  // beyond the fixed scratch
+  float* partial = noalloc_scratch();
+  if (!partial) return TF_ELAUNCH;
+  hipStream_t st = (hipStream_t)stream;
+  // every partial sum the second stage reads is written by the first stage of the same call:
+  // nothing has to start at zero, whatever an earlier (larger) call left behind
   if (dtype == TF_F16) return colsum_launch<f16>(st, rows, cols, x, ldx, out, out_dtype == TF_F32, partial);
   return colsum_launch<bf16>(st, rows, cols, x, ldx, out, out_dtype == TF_F32, partial);
 }
