@@ -121,7 +121,9 @@ def test_attn_large_magnitude_scores(dev):
 
 @pytest.mark.parametrize("dims", [(4, 16, 2048, 64), (2, 16, 2048, 128)])
 def test_baseline_config_shapes(dims, dev):
-    """410M (hd 64) and 1.4B (hd 128) attention shapes at full size; oracle in fp32 on the GPU."""
+    """410M (hd 64) and 1.4B (hd 128) attention shapes at full size, one batch element at a time
+    (keeps the S x S fp32 score matrices small): the first against the fp32 oracle on the CPU, the
+    others against the same oracle expressions evaluated in fp32 on the GPU."""
     b, nh, s, hd = dims
     g = torch.Generator().manual_seed(0)
     raw = [torch.randn(b, s, nh * hd, generator=g).half().to(dev) for _ in range(4)]
@@ -133,10 +135,11 @@ def test_baseline_config_shapes(dims, dev):
     for t in (q, k, v):
         t.grad = None
     worst = 0.0
-    for bi in range(b):  # per batch element: keeps the S x S fp32 score matrix small
-        qr, kr, vr = (t[bi:bi + 1].detach().float().requires_grad_(True) for t in (q, k, v))
+    for bi in range(b):
+        where = "cpu" if bi == 0 else dev
+        qr, kr, vr = (t[bi:bi + 1].detach().float().to(where).requires_grad_(True) for t in (q, k, v))
         orf = R.causal_attention(qr, kr, vr)
-        orf.backward(do[bi:bi + 1].float())
+        orf.backward(do[bi:bi + 1].float().to(where))
         assert_close(o[bi:bi + 1], orf, name="o")
         for got, ref, nm in zip(grads, (qr, kr, vr), "qkv"):
             assert_close(got[bi:bi + 1], ref.grad, name="d" + nm)
