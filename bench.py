@@ -131,7 +131,8 @@ def gemm_table(by_shape, reps, workload, dtype_name):
 
 
 class GemmTimer:
-    """HIP events on the current (launch) stream around every tf_gemm / tf_gemm_relu_bits / tf_gemm_group call."""
+    """HIP events on the current (launch) stream around every tf_gemm / tf_gemm_scaled / tf_gemm_relu_bits /
+    tf_gemm_group call."""
 
     def __init__(self):
         self.records = []
@@ -147,6 +148,16 @@ class GemmTimer:
             e1 = torch.cuda.Event(enable_timing=True)
             e0.record()
             self._orig(dtype, la, lb, m, n, k, *rest, **kw)
+            e1.record()
+            self.records.append(((la, lb, m, n, k), e0, e1))
+
+        self._orig_scaled = kernels._gemm_scaled
+
+        def timed_scaled(dtype, la, lb, m, n, k, *rest):
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record()
+            self._orig_scaled(dtype, la, lb, m, n, k, *rest)
             e1.record()
             self.records.append(((la, lb, m, n, k), e0, e1))
 
@@ -174,12 +185,14 @@ class GemmTimer:
             return rc
 
         kernels._gemm = timed
+        kernels._gemm_scaled = timed_scaled
         kernels._gemm_group = timed_group
         kernels._gemm_bits = timed_bits
         return self
 
     def __exit__(self, *exc):
         self._kernels._gemm = self._orig
+        self._kernels._gemm_scaled = self._orig_scaled
         self._kernels._gemm_group = self._orig_group
         self._kernels._gemm_bits = self._orig_bits
         torch.cuda.synchronize()
@@ -393,7 +406,7 @@ def main():
             "flop_per_launch": round(gflops / launches, 1),
             "avg_launch_us": round(total_ms / launches * 1e3, 2),
             "gemm_ms_per_step": round(total_ms / reps, 3),
-            "measured": f"HIP events on the launch stream around each tf_gemm / tf_gemm_relu_bits / tf_gemm_group call, {reps} instrumented steps "
+            "measured": f"HIP events on the launch stream around each tf_gemm / tf_gemm_scaled / tf_gemm_relu_bits / tf_gemm_group call, {reps} instrumented steps "
                         "run after the timed ones; the event time of a call covers its GEMM kernel(s) and, for a split contraction, "
                         "the reduce kernel; launches = GEMM kernels counted by the library",
         }

@@ -126,6 +126,18 @@ int tf_gemm_relu_bits(void* stream, int dtype, int out_dtype, int layout_a, int 
                       void* C, int64_t ldc, const void* bias,
                       void* bits_out, const void* bits_in, int64_t ld_bits);
 int64_t tf_gemm_workspace_bytes(int layout_a, int layout_b, int64_t M, int64_t N, int64_t K);
+/* C = alpha * (A . B), no bias / ReLU / mask; `alpha`: ONE fp32 value in DEVICE memory, read by
+ * the kernel when it writes its result (applied to the fp32 sums before the rounding to
+ * out_dtype).  For a factor that is itself computed on the GPU: the upstream gradient of the mean
+ * loss divided by the number of rows, which tritonformer/crossentropy.py:24 multiplies into the
+ * (N, V) logits gradient in a pass of its own before the two LM-head gradient products
+ * (transformer.py:330-343) -- here those products take the unscaled gradient and the factor.
+ * Other arguments and the workspace rule as tf_gemm_out. */
+int tf_gemm_scaled(void* stream, int dtype, int out_dtype, int layout_a, int layout_b,
+                   int64_t M, int64_t N, int64_t K,
+                   const void* A, int64_t lda, const void* B, int64_t ldb,
+                   void* C, int64_t ldc, const float* alpha,
+                   void* workspace, int64_t workspace_bytes);
 
 /* `count` (1..4) independent products of one dtype and one pair of operand layouts,
  * no bias / ReLU / mask, each with the arguments of tf_gemm_out_chunked.  When every
@@ -312,6 +324,22 @@ int tf_softmax_bwd(void* stream, int dtype, int64_t rows, int64_t cols,
 int tf_cross_entropy_fwd(void* stream, int dtype, int64_t rows, int64_t V,
                          const void* logits, int64_t ld, int64_t inner_rows, int64_t outer_stride,
                          const int64_t* labels, void* loss, float* lse);
+
+/* tf_cross_entropy_fwd that also writes dlogits[r,v] = (softmax(logits[r,:])[v] - [v == labels[r]])
+ * * grad_scale in the same pass: rows of up to 51200 entries are held in registers between the
+ * log-sum-exp and the gradient, so the logits are read once and the second pass of
+ * tf_cross_entropy_bwd over the (N, V) matrix does not happen (kernels/crossentropy.py:47-75 and
+ * :110-127 as one kernel).  The values equal, bit for bit, tf_cross_entropy_bwd with every
+ * gout[r] = grad_scale (as a value of `dtype`); rows of dlogits are addressed like those of
+ * logits with (ldd, inner_rows, outer_stride_d).  `grad_scale_dev`: one value of `dtype` in device
+ * memory holding grad_scale, used only when the one-kernel form does not apply (longer rows,
+ * unaligned matrices: forward and backward kernels then run one after the other); may be null
+ * otherwise.  grad_scale = 1024 keeps fp16 probabilities of 1e-5 out of the subnormal range. */
+int tf_cross_entropy_fwd_grad(void* stream, int dtype, int64_t rows, int64_t V,
+                              const void* logits, int64_t ld, int64_t inner_rows, int64_t outer_stride,
+                              const int64_t* labels, void* loss, float* lse,
+                              void* dlogits, int64_t ldd, int64_t outer_stride_d,
+                              float grad_scale, const void* grad_scale_dev);
 
 /* dlogits[r,v] = (exp(logits[r,v] - lse[r]) - [v == labels[r]]) * gout[r], rows of
  * dlogits addressed like those of logits with (ldd, inner_rows, outer_stride_d).

@@ -99,6 +99,8 @@ def test_gemm_rejects_bad_arguments():
     assert need > 0 and need % (1024 * 1024 * 4) == 0
     assert g(None, 0, 1, 1, 1024, 1024, 8192, FAKE, 1024, FAKE, 1024, FAKE, 1024, None, 0, None, 0) == -5
     assert lib.tf_gemm_workspace_bytes(0, 1, 8192, 4096, 1024) == 0
+    scaled = lambda alpha: lib.tf_gemm_scaled(None, 0, 0, 0, 1, 64, 64, 64, FAKE, 64, FAKE, 64, FAKE, 64, alpha, None, 0)
+    assert scaled(None) == -1 and scaled(0x1002) == -3     # the factor is a device pointer to one aligned fp32 value
     out_tail = (FAKE, 64, FAKE, 64, FAKE, 64, None, 0, None, 0, None, 0)
     assert lib.tf_gemm_out(None, 0, 1, 0, 1, 64, 64, 64, *out_tail) == -2                       # bf16 out of fp16 in
     assert lib.tf_gemm_out(None, 0, 0, 0, 1, 64, 64, 64, FAKE, 64, FAKE, 64, FAKE, 64, None, 1, FAKE, 64,
@@ -242,6 +244,9 @@ def test_row_kernels_reject_bad_arguments():
     assert lib.tf_softmax_fwd(None, 0, 4, 0, FAKE, 64, FAKE, 64) == -1
     assert lib.tf_cross_entropy_fwd(None, 2, 4, 64, FAKE, 64, 0, 0, FAKE, FAKE, FAKE) == -2
     assert lib.tf_cross_entropy_bwd(None, 0, 4, 64, FAKE, 32, 0, 0, FAKE, FAKE, FAKE, 1, FAKE, 64, 0) == -1
+    assert lib.tf_cross_entropy_fwd_grad(None, 0, 4, 64, FAKE, 64, 0, 0, FAKE, FAKE, FAKE, None, 64, 0, 1.0, None) == -1
+    assert lib.tf_cross_entropy_fwd_grad(None, 0, 4, 64, FAKE, 64, 0, 0, FAKE, FAKE, FAKE, FAKE, 32, 0, 1.0, None) == -1
+    assert lib.tf_cross_entropy_fwd_grad(None, 2, 4, 64, FAKE, 64, 0, 0, FAKE, FAKE, FAKE, FAKE, 64, 0, 1.0, None) == -2
     assert lib.tf_cross_entropy_fwd(None, 0, 6, 64, FAKE, 64, 3, 100, FAKE, FAKE, FAKE) == -1   # groups overlap
     assert lib.tf_colsum(None, 0, 0, 16, 64, FAKE, 64, FAKE, None, 0) == -5
     assert lib.tf_colsum(None, 0, 1, 16, 64, FAKE, 64, FAKE, FAKE, 1 << 20) == -2   # bf16 sums of fp16 input

@@ -8,6 +8,7 @@ from .attention import BiasedCausalAttention as fast_causal_attention_with_bias
 from .attention import CausalAttention as fast_causal_attention
 from .attention import PackedCausalAttention as fast_causal_attention_qkvpacked
 from .crossentropy import CrossEntropyLoss as cross_entropy_loss
+from .crossentropy import LMHeadLoss as lm_head_loss
 from .crossentropy import ShiftedCrossEntropyLoss as shifted_cross_entropy_loss
 from .embedding import EmbeddingSum as embedding_sum
 from .layernorm import AddLayerNorm as add_layer_norm

@@ -30,6 +30,7 @@ SIGNATURES = {
                                  _vp, _i, _vp, _i64, _vp, _i64]),
     "tf_gemm_relu_bits": (_i, [_vp, _i, _i, _i, _i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp,
                                _i64]),
+    "tf_gemm_scaled": (_i, [_vp, _i, _i, _i, _i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _i64]),
     "tf_cast_pack": (_i, [_vp, _i, _i, _i, _i64, _i64, _vp, _i64, _vp, _i64]),
     "tf_embedding_fwd": (_i, [_vp, _i, _i, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _i64, _vp, _i64]),
     "tf_embedding_bwd_workspace_bytes": (_i64, [_i64]),
@@ -57,6 +58,8 @@ SIGNATURES = {
     "tf_softmax_fwd": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _vp, _i64]),
     "tf_softmax_bwd": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64]),
     "tf_cross_entropy_fwd": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _i64, _i64, _vp, _vp, _vp]),
+    "tf_cross_entropy_fwd_grad": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _f,
+                                       _vp]),
     "tf_cross_entropy_bwd": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _i64, _vp, _i64, _i64]),
     "tf_colsum": (_i, [_vp, _i, _i, _i64, _i64, _vp, _i64, _vp, _vp, _i64]),
     "tf_colsum_partial_bytes": (_i64, [_i64, _i64]),

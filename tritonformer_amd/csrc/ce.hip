@@ -105,10 +105,14 @@ __global__ __launch_bounds__(kCeThreads) void ce_fwd(int V, const T* __restrict_
 // Forward for rows that fit into the registers of one workgroup (V <= 8 * NCH * kCeThreads): a
 // thread requests all of its NCH 16-byte chunks at once -- NCH loads in flight instead of four --
 // takes the row maximum first and then the sum of exponentials, both from registers.
-template <typename T, int NCH>
+// GRAD: the same pass also writes (softmax(row) - onehot(label)) * grad_scale to the row of
+// `dlogits` -- the row is still in registers once its log-sum-exp is known, so the gradient of
+// the loss with respect to the logits costs one write instead of a second read-and-write pass.
+template <typename T, int NCH, bool GRAD>
 __global__ __launch_bounds__(kCeThreads) void ce_fwd_regs(int V, const T* __restrict__ logits, RowMap map,
                                                            const int64_t* __restrict__ labels, T* __restrict__ loss,
-                                                           float* __restrict__ lse) {
+                                                           float* __restrict__ lse, T* __restrict__ dlogits,
+                                                           RowMap dmap, float grad_scale) {
   __shared__ float red[2][kCeThreads / 64];
   const int64_t row = blockIdx.x;
   const T* xr = logits + map.at(row);
@@ -154,15 +158,39 @@ __global__ __launch_bounds__(kCeThreads) void ce_fwd_regs(int V, const T* __rest
   for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
   if ((threadIdx.x & 63) == 0) red[1][wave] = s;
   __syncthreads();
-  if (threadIdx.x == 0) {
-    float tot = red[1][0];
+  float tot = red[1][0];
 #pragma unroll
-    for (int w = 1; w < kCeThreads / 64; ++w) tot += red[1][w];
-    const float l = (m2 + log2f(tot)) * kLn2;  // natural-log logsumexp
+  for (int w = 1; w < kCeThreads / 64; ++w) tot += red[1][w];
+  const float l = (m2 + log2f(tot)) * kLn2;  // natural-log logsumexp
+  // back to the log2 domain exactly as the backward kernel does from the stored value: the
+  // gradient written here equals the one ce_bwd would produce, bit for bit
+  const float l2 = l * kLog2e;
+  const int64_t lab = labels[row];
+  if (threadIdx.x == 0) {
     lse[row] = l;
-    const int64_t lab = labels[row];
     const float xl = (lab >= 0 && lab < V) ? (float)xr[lab] : 0.f;
     loss[row] = (T)(l - xl);
+  }
+  if constexpr (GRAD) {
+    T* dr = dlogits + dmap.at(row);
+    const int lab_chunk = (lab >= 0 && lab < V) ? (int)(lab >> 3) : -1;
+#pragma unroll
+    for (int u = 0; u < NCH; ++u) {
+      const int c = threadIdx.x + u * kCeThreads;
+      if (c < nchunk) {
+        float v[8];
+        unpack8<T>(raw[u], v);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = fast_exp2(v[e] * kLog2e - l2);
+        if (c == lab_chunk) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[e] -= (e == (int)(lab & 7)) ? 1.0f : 0.0f;
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] *= grad_scale;
+        Chunk<T>::store(dr + c * 8, v);
+      }
+    }
   }
 }
 
@@ -205,16 +233,16 @@ template <typename T>
 static int ce_fwd_launch(hipStream_t st, int64_t rows, int64_t V, const void* logits, RowMap map,
                          const int64_t* labels, void* loss, float* lse) {
   const dim3 grid((unsigned)rows), block(kCeThreads);
+  const RowMap none = {0, 0, 1};
   if (row_vectorizable<T>(logits, V, map.ld) && map.outer % 8 == 0) {
     const int64_t per_thread = (V / 8 + kCeThreads - 1) / kCeThreads;  // 16-byte chunks per thread
-    if (per_thread <= 8)
-      ce_fwd_regs<T, 8><<<grid, block, 0, st>>>((int)V, (const T*)logits, map, labels, (T*)loss, lse);
-    else if (per_thread <= 16)
-      ce_fwd_regs<T, 16><<<grid, block, 0, st>>>((int)V, (const T*)logits, map, labels, (T*)loss, lse);
-    else if (per_thread <= 25)
-      ce_fwd_regs<T, 25><<<grid, block, 0, st>>>((int)V, (const T*)logits, map, labels, (T*)loss, lse);
-    else
-      ce_fwd<T, true><<<grid, block, 0, st>>>((int)V, (const T*)logits, map, labels, (T*)loss, lse);
+#define CE_REGS(NCH) \
+  ce_fwd_regs<T, NCH, false><<<grid, block, 0, st>>>((int)V, (const T*)logits, map, labels, (T*)loss, lse, nullptr, none, 0.f)
+    if (per_thread <= 8) CE_REGS(8);
+    else if (per_thread <= 16) CE_REGS(16);
+    else if (per_thread <= 25) CE_REGS(25);
+    else ce_fwd<T, true><<<grid, block, 0, st>>>((int)V, (const T*)logits, map, labels, (T*)loss, lse);
+#undef CE_REGS
   } else
     ce_fwd<T, false><<<grid, block, 0, st>>>((int)V, (const T*)logits, map, labels, (T*)loss, lse);
   TF_CHECK_LAUNCH();
@@ -235,6 +263,34 @@ static int ce_bwd_launch(hipStream_t st, int64_t rows, int64_t V, const void* lo
                                              (T*)dlogits, dmap);
   TF_CHECK_LAUNCH();
   return TF_OK;
+}
+
+// Forward that also leaves (softmax - onehot) * grad_scale in dlogits: one kernel when the row fits
+// the registers of a workgroup and both matrices can be accessed in 16-byte chunks, else the forward
+// followed by the backward kernel with `scale_dev` (one value of T in device memory holding
+// grad_scale) as the upstream gradient of every row -- the same values either way.
+template <typename T>
+static int ce_fwd_grad_launch(hipStream_t st, int64_t rows, int64_t V, const void* logits, RowMap map,
+                              const int64_t* labels, void* loss, float* lse, void* dlogits, RowMap dmap,
+                              float grad_scale, const void* scale_dev) {
+  const dim3 grid((unsigned)rows), block(kCeThreads);
+  const int64_t per_thread = (V / 8 + kCeThreads - 1) / kCeThreads;
+  if (row_vectorizable<T>(logits, V, map.ld) && map.outer % 8 == 0 && row_vectorizable<T>(dlogits, V, dmap.ld) &&
+      dmap.outer % 8 == 0 && per_thread <= 25) {
+#define CE_REGS(NCH)                                                                                               \
+  ce_fwd_regs<T, NCH, true><<<grid, block, 0, st>>>((int)V, (const T*)logits, map, labels, (T*)loss, lse, (T*)dlogits, \
+                                                    dmap, grad_scale)
+    if (per_thread <= 8) CE_REGS(8);
+    else if (per_thread <= 16) CE_REGS(16);
+    else CE_REGS(25);
+#undef CE_REGS
+    TF_CHECK_LAUNCH();
+    return TF_OK;
+  }
+  if (!scale_dev) return TF_EINVAL;
+  const int rc = ce_fwd_launch<T>(st, rows, V, logits, map, labels, loss, lse);
+  if (rc != TF_OK) return rc;
+  return ce_bwd_launch<T>(st, rows, V, logits, map, labels, lse, scale_dev, 0, dlogits, dmap);
 }
 
 }  // namespace tfa
@@ -278,4 +334,21 @@ extern "C" int tf_cross_entropy_bwd(void* stream, int dtype, int64_t rows, int64
   if (dtype == TF_BF16)
     return ce_bwd_launch<bf16>(st, rows, V, logits, map, labels, lse, gout, gout_stride, dlogits, dmap);
   return TF_EDTYPE;
+}
+
+extern "C" int tf_cross_entropy_fwd_grad(void* stream, int dtype, int64_t rows, int64_t V, const void* logits,
+                                         int64_t ld, int64_t inner_rows, int64_t outer_stride, const int64_t* labels,
+                                         void* loss, float* lse, void* dlogits, int64_t ldd, int64_t outer_stride_d,
+                                         float grad_scale, const void* grad_scale_dev) {
+  if (!logits || !labels || !loss || !lse || !dlogits) return TF_EINVAL;
+  if (rows < 0 || rows > 0x7fffffff || V <= 0 || V > (1 << 30)) return TF_EINVAL;
+  RowMap map, dmap;
+  if (!make_map(map, rows, V, ld, inner_rows, outer_stride)) return TF_EINVAL;
+  if (!make_map(dmap, rows, V, ldd, inner_rows, outer_stride_d)) return TF_EINVAL;
+  if (dtype != TF_F16 && dtype != TF_BF16) return TF_EDTYPE;
+  if (rows == 0) return TF_OK;
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == TF_F16)
+    return ce_fwd_grad_launch<f16>(st, rows, V, logits, map, labels, loss, lse, dlogits, dmap, grad_scale, grad_scale_dev);
+  return ce_fwd_grad_launch<bf16>(st, rows, V, logits, map, labels, loss, lse, dlogits, dmap, grad_scale, grad_scale_dev);
 }

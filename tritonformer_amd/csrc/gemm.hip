@@ -64,6 +64,10 @@ struct GemmParams {
   // One matrix: chunk_n = N, chunk_skip = 0.
   int chunk_n;
   int64_t chunk_skip;
+  // Optional factor on the whole product, one fp32 value in DEVICE memory (null = 1): it is applied
+  // to the fp32 sums before bias / rounding.  A pointer, so that a value computed on the GPU (the
+  // upstream gradient of a mean loss) needs no host round trip.
+  const float* alpha;
 };
 
 __device__ __forceinline__ int64_t c_index(const GemmParams& p, int m, int n) {
@@ -157,6 +161,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                                               int wn, int lane, int split) {
   const T* bias = (const T*)p.bias;
   T* C = (T*)p.C;
+  const float alpha = (p.alpha && p.splits <= 1) ? *p.alpha : 1.f;  // a split contraction is scaled by its reduce pass
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     const int m = m0 + wm * WTM + i * 32 + (lane & 31);
@@ -169,7 +174,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
         if (n >= p.N) continue;
         float v[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = acc[i][j][g * 4 + e];
+        for (int e = 0; e < 4; ++e) v[e] = acc[i][j][g * 4 + e] * alpha;
         if (p.splits > 1) {
           float* dst = p.partial + ((int64_t)split * p.M + m) * p.N + n;
           if (VEC) {
@@ -433,6 +438,7 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x16 (&
   const void* mask = PLAIN ? nullptr : p.mask;
   const void* sign_in = PLAIN ? nullptr : p.sign_in;
   void* sign_out = PLAIN ? nullptr : p.sign_out;
+  const float alpha = (!PLAIN && p.alpha) ? *p.alpha : 1.f;
   TO* C = (TO*)p.C;
   const int nbase = n0 + wn * WTN;
   // this lane stores the same 16-byte column chunk of every row it handles: the column part of the
@@ -461,6 +467,10 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x16 (&
         float v[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[e] = acc[i][j][g * 4 + e];
+        if (!PLAIN) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] *= alpha;
+        }
         if (bias) {
 #pragma unroll
           for (int e = 0; e < 4; ++e) v[e] += (float)bvals[j][g][e];
@@ -689,13 +699,14 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams& p, const int pid
     q.mask = nullptr;
     q.sign_out = nullptr;
     q.sign_in = nullptr;
+    q.alpha = nullptr;
     q.chunk_n = p.N;
     q.chunk_skip = 0;
     __syncthreads();  // all waves are done reading the last pipeline stage
     gemm_epilogue_lds<T, float, TM, TN, WTM, WTN, true>(q, acc, smem, m0, n0, wm, wn, wave, lane);
   } else {
     __syncthreads();  // all waves are done reading the last pipeline stage
-    const bool plain = !p.bias && !p.relu && !p.mask && !p.sign_in && !p.sign_out;
+    const bool plain = !p.bias && !p.relu && !p.mask && !p.sign_in && !p.sign_out && !p.alpha;
     if (p.out_f32) {
       if (plain) gemm_epilogue_lds<T, float, TM, TN, WTM, WTN, true>(p, acc, smem, m0, n0, wm, wn, wave, lane);
       else gemm_epilogue_lds<T, float, TM, TN, WTM, WTN>(p, acc, smem, m0, n0, wm, wn, wave, lane);
@@ -736,8 +747,10 @@ __global__ __launch_bounds__(WM* WN * 64, WPE) void gemm_dma_group_kernel(GemmGr
 template <typename T, typename TO, bool VEC4>
 __global__ __launch_bounds__(256) void gemm_reduce(int M, int N, int splits, const float* __restrict__ partial,
                                                     const T* __restrict__ bias, int relu, TO* __restrict__ C,
-                                                    int64_t ldc, int chunk_n, int64_t chunk_skip) {
+                                                    int64_t ldc, int chunk_n, int64_t chunk_skip,
+                                                    const float* __restrict__ alpha_ptr) {
   const int64_t total = (int64_t)M * N;
+  const float alpha = alpha_ptr ? *alpha_ptr : 1.f;
   if (VEC4) {
     const int64_t quads = total >> 2;
     for (int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x; q < quads; q += (int64_t)gridDim.x * 256) {
@@ -748,7 +761,7 @@ __global__ __launch_bounds__(256) void gemm_reduce(int M, int N, int splits, con
       TO o[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        float x = s[e] + (bias ? (float)bias[n + e] : 0.f);
+        float x = s[e] * alpha + (bias ? (float)bias[n + e] : 0.f);
         o[e] = (TO)(relu ? fmaxf(x, 0.f) : x);
       }
       struct alignas(sizeof(TO) * 4) Quad { TO v[4]; };
@@ -762,6 +775,7 @@ __global__ __launch_bounds__(256) void gemm_reduce(int M, int N, int splits, con
       float s = 0.f;
       for (int k = 0; k < splits; ++k) s += partial[(int64_t)k * total + i];
       const int m = (int)(i / N), n = (int)(i - (int64_t)m * N);
+      s *= alpha;
       if (bias) s += (float)bias[n];
       C[(int64_t)m * ldc + n + (int64_t)(n / chunk_n) * chunk_skip] = (TO)(relu ? fmaxf(s, 0.f) : s);
     }
@@ -977,7 +991,7 @@ static int launch_reduce(hipStream_t st, const GemmParams& p) {
   const T* bias = (const T*)p.bias;
 #define REDUCE(TO, V4) \
   gemm_reduce<T, TO, V4><<<g, b, 0, st>>>(p.M, p.N, p.splits, p.partial, bias, p.relu, (TO*)p.C, p.ldc, p.chunk_n, \
-                                          p.chunk_skip)
+                                          p.chunk_skip, p.alpha)
   if (p.out_f32) { if (v4) REDUCE(float, true); else REDUCE(float, false); }
   else { if (v4) REDUCE(T, true); else REDUCE(T, false); }
 #undef REDUCE
@@ -1136,8 +1150,9 @@ static int gemm_entry(void* stream, int dtype, int out_dtype, int layout_a, int 
                       int64_t K, const void* A, int64_t lda, const void* B, int64_t ldb, void* C, int64_t ldc,
                       int64_t chunk_n, int64_t chunk_stride, const void* bias, int relu, const void* mask_act,
                       int64_t ld_mask, void* workspace, int64_t workspace_bytes, void* sign_out, const void* sign_in,
-                      int64_t ld_sign, const GemmForce& force = kNoForce) {
+                      int64_t ld_sign, const GemmForce& force = kNoForce, const float* alpha = nullptr) {
   if (!A || !B || !C) return TF_EINVAL;
+  if (alpha && (reinterpret_cast<uintptr_t>(alpha) & 3)) return TF_EALIGN;
   const bool signs = sign_out || sign_in;
   if (signs) {
     if ((sign_out && sign_in) || mask_act || N % 8 != 0 || ld_sign < N / 8 || (chunk_n != 0 && chunk_n < N)) return TF_EINVAL;
@@ -1174,10 +1189,11 @@ static int gemm_entry(void* stream, int dtype, int out_dtype, int layout_a, int 
       const void* bias2 = bias ? (const char*)bias + n1 * 2 : nullptr;
       const void* mask2 = mask_act ? (const char*)mask_act + n1 * 2 : nullptr;
       const int rc = gemm_entry(stream, dtype, out_dtype, layout_a, layout_b, M, n1, K, A, lda, B, ldb, C, ldc, 0, 0, bias,
-                                relu, mask_act, ld_mask, workspace, workspace_bytes, nullptr, nullptr, 0, force);
+                                relu, mask_act, ld_mask, workspace, workspace_bytes, nullptr, nullptr, 0, force, alpha);
       if (rc != TF_OK) return rc;
       return gemm_entry(stream, dtype, out_dtype, layout_a, layout_b, M, tail, K, A, lda, b2, ldb, (char*)C + n1 * osz,
-                        ldc, 0, 0, bias2, relu, mask2, ld_mask, workspace, workspace_bytes, nullptr, nullptr, 0, force);
+                        ldc, 0, 0, bias2, relu, mask2, ld_mask, workspace, workspace_bytes, nullptr, nullptr, 0, force,
+                        alpha);
     }
   }
   const GemmPlan pl = make_plan(M, N, K, vec, mask_act == nullptr && !signs, nullptr, force);
@@ -1205,6 +1221,7 @@ static int gemm_entry(void* stream, int dtype, int out_dtype, int layout_a, int 
   p.ldsign = ld_sign;
   p.chunk_n = (int)chunk_n;
   p.chunk_skip = chunk_stride - chunk_n;
+  p.alpha = alpha;
   hipStream_t st = (hipStream_t)stream;
   if (dtype == TF_F16) return gemm_dispatch<f16>(st, layout_a, layout_b, vec, pl, p);
   return gemm_dispatch<bf16>(st, layout_a, layout_b, vec, pl, p);
@@ -1226,6 +1243,14 @@ extern "C" int tf_gemm_relu_bits(void* stream, int dtype, int out_dtype, int lay
   if (!bits_out && !bits_in) return TF_EINVAL;
   return gemm_entry(stream, dtype, out_dtype, layout_a, layout_b, M, N, K, A, lda, B, ldb, C, ldc, 0, 0, bias,
                     bits_out ? 1 : 0, nullptr, 0, nullptr, 0, bits_out, bits_in, ld_bits);
+}
+
+extern "C" int tf_gemm_scaled(void* stream, int dtype, int out_dtype, int layout_a, int layout_b, int64_t M, int64_t N,
+                              int64_t K, const void* A, int64_t lda, const void* B, int64_t ldb, void* C, int64_t ldc,
+                              const float* alpha, void* workspace, int64_t workspace_bytes) {
+  if (!alpha) return TF_EINVAL;
+  return gemm_entry(stream, dtype, out_dtype, layout_a, layout_b, M, N, K, A, lda, B, ldb, C, ldc, 0, 0, nullptr, 0,
+                    nullptr, 0, workspace, workspace_bytes, nullptr, nullptr, 0, kNoForce, alpha);
 }
 
 // Diagnostic twin of tf_gemm_out_chunked: the same call with a tile configuration, a contraction
@@ -1359,6 +1384,7 @@ extern "C" int tf_gemm_group(void* stream, int dtype, int out_dtype, int layout_
     p.sign_out = nullptr; p.sign_in = nullptr; p.ldsign = 0;
     p.chunk_n = (int)cn;
     p.chunk_skip = (cn == q.N ? q.N : q.chunk_stride) - cn;
+    p.alpha = nullptr;
     if (i < count) {
       g.first[i + 1] = g.first[i] + p.tiles_m * p.tiles_n * p.splits;
       if (p.splits > 1) ws += (int64_t)gp.splits * q.M * q.N * (int64_t)sizeof(float);

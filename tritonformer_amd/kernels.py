@@ -147,6 +147,25 @@ def mm_masked_bits(a, b, bits, act=None):
     return out
 
 
+def _gemm_scaled(dtype, la, lb, m, n, k, a, lda, b, ldb, c, ldc, alpha):
+    lib = load()
+    ws_bytes = _gemm_ws(la, lb, m, n, k)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=c.device) if ws_bytes else None
+    check(lib.tf_gemm_scaled(stream_ptr(), dtype_code(dtype), dtype_code(c.dtype), la, lb, m, n, k, a.data_ptr(), lda,
+                             b.data_ptr(), ldb, c.data_ptr(), ldc, alpha.data_ptr(),
+                             ws.data_ptr() if ws is not None else None, ws_bytes))
+
+
+def gemm_scaled(a, la, m, k, lda, b, lb, n, ldb, alpha, out):
+    """``out (m, n) = alpha * A . B`` through tf_gemm_scaled; ``alpha``: a one-element float32 tensor on
+    the GPU; operands given with their layouts as in the C header.  ``out``: float32 or the operand dtype."""
+    if alpha.dtype != torch.float32 or alpha.numel() != 1:
+        raise TypeError("alpha must be a one-element float32 tensor")
+    require_cuda(a, b, alpha, out)
+    _gemm_scaled(a.dtype, la, lb, m, n, k, a, lda, b, ldb, out, out.stride(0), alpha)
+    return out
+
+
 def mm(a, b, fuse_relu=False, mask_act=None):
     return gemm(a, b, None, fuse_relu, mask_act)
 
@@ -644,6 +663,31 @@ def shifted_cross_entropy_fwd(logits, labels):
     check(load().tf_cross_entropy_fwd(stream_ptr(), dtype_code(logits.dtype), n, v, logits.data_ptr(), v, s - 1,
                                       s * v, shift_labels.data_ptr(), loss.data_ptr(), lse.data_ptr()))
     return loss, lse, logits, shift_labels
+
+
+def shifted_cross_entropy_fwd_grad(logits, labels, grad_scale):
+    """shifted_cross_entropy_fwd that also returns ``(softmax - onehot) * grad_scale`` for every row,
+    as a (B, S, V) tensor whose last position per sequence is zero, written by the same kernel pass
+    (reference kernels/crossentropy.py:47-75 and :110-127 in one).  ``grad_scale`` must be exactly
+    representable in the logits' dtype (a power of two).
+    -> (loss (B*(S-1),), lse, dlogits)"""
+    if logits.ndim != 3 or labels.shape != logits.shape[:2]:
+        raise ValueError("shifted cross entropy takes (B, S, V) logits and (B, S) labels")
+    _check_ce(logits, labels)
+    if not logits.is_contiguous():
+        logits = logits.contiguous()
+    b, s, v = logits.shape
+    shift_labels = labels[:, 1:].contiguous().view(-1)
+    n = b * (s - 1)
+    loss = torch.empty((n,), dtype=logits.dtype, device=logits.device)
+    lse = torch.empty((n,), dtype=torch.float32, device=logits.device)
+    dlogits = torch.empty((b, s, v), dtype=logits.dtype, device=logits.device)
+    dlogits[:, -1].zero_()
+    scale_dev = torch.full((1,), grad_scale, dtype=logits.dtype, device=logits.device)
+    check(load().tf_cross_entropy_fwd_grad(stream_ptr(), dtype_code(logits.dtype), n, v, logits.data_ptr(), v, s - 1,
+                                           s * v, shift_labels.data_ptr(), loss.data_ptr(), lse.data_ptr(),
+                                           dlogits.data_ptr(), v, s * v, float(grad_scale), scale_dev.data_ptr()))
+    return loss, lse, dlogits
 
 
 def shifted_cross_entropy_bwd(grad_out, logits, shift_labels, lse):

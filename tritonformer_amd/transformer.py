@@ -26,6 +26,7 @@ from . import (
     fast_causal_attention_qkvpacked,
     fast_causal_attention_with_bias,
     linear_no_bias_packed,
+    lm_head_loss,
     mlp_fused_relu,
     shifted_cross_entropy_loss,
 )
@@ -90,6 +91,11 @@ FUSE_ADD_LN = True
 # one kernel, and the table gradients a chain-ordered scatter-add; False: two nn.Embedding
 # calls and an addition as in the reference (transformer.py:311-323).
 FUSE_EMBED = True
+# True: LM head, shifted cross-entropy and the mean are one autograd node -- the cross-entropy forward
+# writes the logits gradient in the pass that reads the logits, and the 1/N of the mean rides on the
+# write-out of the two LM-head gradient GEMMs; False: logits_out module, shifted_cross_entropy_loss
+# and .mean() one after the other (the reference's sequence, transformer.py:330-343).
+FUSE_HEAD = True
 # True (read when a model with attn_bias=True is built): no dense (nh, S, S) ALiBi matrix --
 # 805 MB at 24 heads x 4096 -- is made; the attention kernels compute -slope_h * (i - j) from
 # the nh slopes with the roundings of that matrix, bit-identical results.  False: the dense
@@ -281,7 +287,11 @@ class Transformer(nn.Module):
             for layer in self.layer_list:
                 hidden_states = layer(hidden_states, attn_bias)
             hidden_states = self.final_layernorm(hidden_states)
-        logits_lm = self.logits_out(hidden_states)
+        head = self.logits_out
+        if (FUSE_HEAD and labels is not None and isinstance(head, tnn.Linear) and head.bias is None
+                and not head.fuse_activation and hidden_states.is_cuda):
+            return lm_head_loss.apply(hidden_states, head.weight, labels)   # (logits, mean shifted loss)
+        logits_lm = head(hidden_states)
         if labels is None:
             return logits_lm
         # same rows and labels as the reference's shift-copy-then-cross-entropy
