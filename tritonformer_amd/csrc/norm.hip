@@ -7,6 +7,10 @@
 namespace tfa {
 
 constexpr int kRowsPerBlock = 4;  // 4 waves per workgroup, one row each
+#ifndef TF_LN_FWD_ROWS
+#define TF_LN_FWD_ROWS 2
+#endif
+constexpr int kLnFwdRowsPerWave = TF_LN_FWD_ROWS;  // rows a wave of the forward kernel walks (with the next one in flight)
 
 // ---------------------------------------------------------------------------
 // LayerNorm forward.  NV = 16-byte chunks per lane (row length <= NV*64*8).
@@ -21,57 +25,76 @@ __global__ __launch_bounds__(256) void ln_fwd_vec(int64_t rows, int d, const T* 
                                                    const TP* __restrict__ gamma, const TP* __restrict__ beta,
                                                    float eps, T* __restrict__ y, int64_t ldy,
                                                    float* __restrict__ mean_out, float* __restrict__ rstd_out) {
+  // Wave w of workgroup b walks rows (b*4 + w) + k*4*grid.  The raw chunks of the wave's next row
+  // are requested before the cross-lane sums of the current one, so that the reads of one row run
+  // beside the reductions and the stores of the row before: with one row per wave and every wave
+  // of the launch resident at once, the whole launch reads first and writes afterwards, and
+  // neither half of the memory system's time is used by the other.
   const int lane = threadIdx.x & 63;
-  const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
-  if (row >= rows) return;
   const int nchunk = d >> 3;
-  const T* xr = x + row * ldx;
-  float v[NV][8];
-  float s = 0.f;
+  const int64_t stride = (int64_t)gridDim.x * kRowsPerBlock;
+  u32x4 raw_x[NV], raw_r[ADD ? NV : 1];
+  auto fetch = [&](int64_t row) {
 #pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    const int c = lane + i * 64;
-    if (c < nchunk) {
-      Chunk<T>::load(xr + c * 8, v[i]);
-      if (ADD) {
-        float r[8];
-        Chunk<T>::load(res + row * ldres + c * 8, r);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) v[i][e] += r[e];
-        const u32x4 packed = pack8<T>(v[i]);
-        st16(sum + row * ldsum + c * 8, packed);
-        unpack8<T>(packed, v[i]);
+    for (int i = 0; i < NV; ++i) {
+      const int c = lane + i * 64;
+      if (c < nchunk) {
+        raw_x[i] = ld16(x + row * ldx + c * 8);
+        if (ADD) raw_r[i] = ld16(res + row * ldres + c * 8);
       }
-#pragma unroll
-      for (int e = 0; e < 8; ++e) s += v[i][e];
-    } else {
-#pragma unroll
-      for (int e = 0; e < 8; ++e) v[i][e] = 0.f;
     }
-  }
-  const float mean = wave_sum(s) / (float)d;
-  float q = 0.f;
+  };
+  int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
+  if (row < rows) fetch(row);
+  for (; row < rows; row += stride) {
+    float v[NV][8];
+    float s = 0.f;
 #pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    if (lane + i * 64 < nchunk) {
+    for (int i = 0; i < NV; ++i) {
+      const int c = lane + i * 64;
+      if (c < nchunk) {
+        unpack8<T>(raw_x[i], v[i]);
+        if (ADD) {
+          float r[8];
+          unpack8<T>(raw_r[i], r);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) { const float t = v[i][e] - mean; q += t * t; }
+          for (int e = 0; e < 8; ++e) v[i][e] += r[e];
+          const u32x4 packed = pack8<T>(v[i]);
+          st16(sum + row * ldsum + c * 8, packed);
+          unpack8<T>(packed, v[i]);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s += v[i][e];
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[i][e] = 0.f;
+      }
     }
-  }
-  const float var = wave_sum(q) / (float)d;
-  const float rstd = 1.0f / sqrtf(var + eps);
-  if (lane == 0) { mean_out[row] = mean; rstd_out[row] = rstd; }
-  T* yr = y + row * ldy;
+    if (row + stride < rows) fetch(row + stride);
+    const float mean = wave_sum(s) / (float)d;
+    float q = 0.f;
 #pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    const int c = lane + i * 64;
-    if (c < nchunk) {
-      float g[8], b[8], o[8];
-      load8<TP>(gamma + c * 8, g);
-      load8<TP>(beta + c * 8, b);
+    for (int i = 0; i < NV; ++i) {
+      if (lane + i * 64 < nchunk) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) o[e] = (v[i][e] - mean) * rstd * g[e] + b[e];
-      Chunk<T>::store(yr + c * 8, o);
+        for (int e = 0; e < 8; ++e) { const float t = v[i][e] - mean; q += t * t; }
+      }
+    }
+    const float var = wave_sum(q) / (float)d;
+    const float rstd = 1.0f / sqrtf(var + eps);
+    if (lane == 0) { mean_out[row] = mean; rstd_out[row] = rstd; }
+    T* yr = y + row * ldy;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int c = lane + i * 64;
+      if (c < nchunk) {
+        float g[8], b[8], o[8];
+        load8<TP>(gamma + c * 8, g);
+        load8<TP>(beta + c * 8, b);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = (v[i][e] - mean) * rstd * g[e] + b[e];
+        Chunk<T>::store(yr + c * 8, o);
+      }
     }
   }
 }
@@ -424,8 +447,13 @@ static int ln_fwd_launch(hipStream_t st, int64_t rows, int64_t d, const void* x,
   bool vec = row_vectorizable<T>(x, d, ldx) && row_vectorizable<T>(y, d, ldy) && aligned16(gamma) && aligned16(beta);
   if (ADD) vec = vec && row_vectorizable<T>(res, d, ldres) && row_vectorizable<T>(sum, d, ldsum);
   const int nv = vec ? pick_nv(d / 8) : 0;
+  // the row-walking kernel: kLnFwdRowsPerWave rows per wave once there are enough rows to fill the chip
+  int64_t walkers = ceil_div(rows, kRowsPerBlock * kLnFwdRowsPerWave);
+  const int64_t fill = (int64_t)device_shape().cus * 4;
+  if (walkers < fill) walkers = ceil_div(rows, kRowsPerBlock) < fill ? ceil_div(rows, kRowsPerBlock) : fill;
+  const dim3 wgrid((unsigned)walkers);
 #define LN_FWD(NV)                                                                                             \
-  ln_fwd_vec<T, TP, NV, ADD><<<grid, block, 0, st>>>(rows, (int)d, (const T*)x, ldx, (const T*)res, ldres, (T*)sum, \
+  ln_fwd_vec<T, TP, NV, ADD><<<wgrid, block, 0, st>>>(rows, (int)d, (const T*)x, ldx, (const T*)res, ldres, (T*)sum, \
                                                      ldsum, (const TP*)gamma, (const TP*)beta, eps, (T*)y, ldy, mean, \
                                                      rstd)
   switch (nv) {
