@@ -565,7 +565,7 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams& p, const int pid
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: LDS slab addresses stay scalar
   const int wm = wave / WN, wn = wave % WN;
 
   const int tiles = p.tiles_m * p.tiles_n;
