@@ -29,11 +29,9 @@
 #include <atomic>
 #include <cstdio>
 #include <cstdlib>
+#include <type_traits>
 #include "rowops.h"
 
-#ifndef TF_GEMM_NSLICE
-#define TF_GEMM_NSLICE 2  // the loads of the next step go out in this many slices, early in the step
-#endif
 
 namespace tfa {
 
@@ -559,8 +557,8 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams& p, const int pid
   typedef typename Vec<T>::v8 v8;
   constexpr int STAGE = PA::BYTES + PB::BYTES;      // two stages, ping-pong
   constexpr int LPS = PA::PER_WAVE + PB::PER_WAVE;  // loads per wave per stage
-  constexpr int NREAD = TM * PA::READS_PER_FRAG + TN * PB::READS_PER_FRAG;  // LDS reads per contraction step
-  static_assert(NREAD <= 15, "lgkmcnt range");
+  constexpr int NEARLY = LPS / 2;  // loads of a stage issued right after the hand-over to the stage before it
+  static_assert(KSTEPS >= 3, "the loop deals its loads and pointer updates over the first two steps and the last one");
   static_assert(KSTEPS % 2 == 0, "operand register ping-pong needs an even number of contraction steps");
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
@@ -618,18 +616,6 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams& p, const int pid
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
   };
-  // slice sl (of NSLICE) of this wave's loads of one contraction step, into stage `dst`;
-  // slices >= NSLICE are empty
-  constexpr int NSLICE = TF_GEMM_NSLICE < KSTEPS ? TF_GEMM_NSLICE : KSTEPS;
-  auto issue_slice = [&](char* dst, int sl) {
-#pragma unroll
-    for (int q = 0; q < LPS; ++q) {
-      if (q * NSLICE / LPS == sl) {
-        if (q < PA::PER_WAVE) PA::issue_one(pa, dst, wave, q);
-        else PB::issue_one(pb, dst + PA::BYTES, wave, q - PA::PER_WAVE);
-      }
-    }
-  };
   FragRegs<A_KMAJOR> fa[2][TM];
   FragRegs<B_KMAJOR> fb[2][TN];
   auto read_operands = [&](const char* stage, int ks, int buf) {
@@ -649,44 +635,94 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams& p, const int pid
     wait_vmcnt<0>();
     barrier();
     read_operands(smem, 0, 0);
-    if (nk > 1) issue_slice(smem + STAGE, 0);
-  }
-
-  // ---- main loop.  Per step of BK: the operands of contraction step ks+1 are requested
-  // from LDS before the MFMAs of step ks are issued; the loads of the next BK step
-  // trickle in slice by slice; and the hand-over to the next stage (wait for the loads,
-  // barrier, first operand reads of the next stage, head of the step after) happens
-  // BEFORE the last group of MFMAs, so no MFMA ever waits on a freshly issued LDS read.
-  for (int kt = 0; kt < nk; ++kt) {
-    char* cur = smem + (kt & 1) * STAGE;
-    char* nxt = smem + ((kt + 1) & 1) * STAGE;
-    const bool more = kt + 1 < nk;
+    if (nk > 1) {
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) {
-      if (ks + 1 < KSTEPS) {
-        read_operands(cur, ks + 1, (ks + 1) & 1);
-        wait_lgkmcnt<NREAD>();  // step ks has landed; step ks+1 may still be in flight
-        if (more) issue_slice(nxt, ks + 1);
-      } else {
-        wait_lgkmcnt<0>();      // every LDS read of this stage is complete
-        if (more) {
-          PA::advance(pa, p.lda);
-          PB::advance(pb, p.ldb);
-          wait_vmcnt<0>();      // this wave's loads of the next stage have landed
-          barrier();            // ... and everyone's; everyone is done reading `cur`
-          read_operands(nxt, 0, 0);
-          if (kt + 2 < nk) issue_slice(cur, 0);
-        }
+      for (int q = 0; q < NEARLY; ++q) {
+        if (q < PA::PER_WAVE) PA::issue_one(pa, smem + STAGE, wave, q);
+        else PB::issue_one(pb, smem + STAGE + PA::BYTES, wave, q - PA::PER_WAVE);
       }
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc[i][j] = mfma32(fb[ks & 1][j].template get<v8>(), fa[ks & 1][i].template get<v8>(), acc[i][j]);
-      __builtin_amdgcn_sched_barrier(0);
     }
   }
+
+  // ---- main loop.  Every LDS read, load and pointer update sits behind an MFMA, pinned there by
+  // scheduling barriers: the matrix pipe is busy for 32 cycles per MFMA and the wave is free to
+  // issue meanwhile.  Per 16-wide step there are NMFMA slots; the operand reads of the next step
+  // go behind the first ones (register ping-pong: the MFMAs of step ks read set ks % 2), the extras
+  // of the step behind the rest -- half of the next stage's loads at step 0, the pointer updates
+  // at step 1, and in the last step the hand-over (wait for this wave's loads, barrier) followed
+  // by the first operand reads of the next stage and the other half of the loads, which go into
+  // the buffer everyone has just left.
+  constexpr int NMFMA = TM * TN;
+  constexpr int NR = TM + TN;                                       // read items (one fragment each)
+  constexpr int RPS = (NR + NMFMA - 1) / NMFMA;                     // read items per slot
+  constexpr int RSLOTS = (NR + RPS - 1) / RPS;                      // slots that carry reads
+  constexpr int HAND = NMFMA - RSLOTS >= 4 ? 2 : 0;                 // MFMAs of the last step ahead of the barrier
+  static_assert(HAND + RSLOTS <= NMFMA, "the reads of a step must fit behind its MFMAs");
+  static_assert(LPS % 2 == 0, "loads go out in two halves");
+  auto read_item = [&](const char* stage, int ks, int buf, int item) {
+    const uint32_t sa_addr = lds_address(stage), sb_addr = sa_addr + PA::BYTES;
+    if (item < TM) PA::frag_issue(fa[buf][item], sa_addr, wm * WTM + item * 32, ks, lane);
+    else PB::frag_issue(fb[buf][item - TM], sb_addr, wn * WTN + (item - TM) * 32, ks, lane);
+  };
+  auto load_item = [&](char* dst, int q) {
+    if (q < PA::PER_WAVE) PA::issue_one(pa, dst, wave, q);
+    else PB::issue_one(pb, dst + PA::BYTES, wave, q - PA::PER_WAVE);
+  };
+  auto advance_item = [&](int q) {
+    if (q < PA::PER_WAVE) pa[q] += A_KMAJOR ? (int64_t)BK : (int64_t)BK * p.lda;
+    else pb[q - PA::PER_WAVE] += B_KMAJOR ? (int64_t)BK : (int64_t)BK * p.ldb;
+  };
+  // One 64-wide stage.  MORE: another stage follows (hand over to it); MORE2: and one after that
+  // (its first loads go out).  Compile-time, so the steady state of the loop has no branch.
+  auto stage = [&](char* cur, char* nxt, auto more_c, auto more2_c) {
+    constexpr bool MORE = decltype(more_c)::value, MORE2 = decltype(more2_c)::value;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      const bool last = ks + 1 == KSTEPS;
+      const int first = last ? HAND : 0;                 // first slot that carries work of this step
+      const int xfirst = first + RSLOTS < NMFMA ? first + RSLOTS : NMFMA - 1;  // extras: behind the reads
+      const int xslots = NMFMA - xfirst;
+      const int nx = !MORE ? 0 : last ? (MORE2 ? NEARLY : 0) : ks == 0 ? LPS - NEARLY : ks == 1 ? LPS : 0;
+      wait_lgkmcnt<0>();  // the operands of this step were requested a whole step ago
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int m = 0; m < NMFMA; ++m) {
+        const int i = m / TN, j = m % TN;
+        if (last && m == HAND && MORE) {
+          wait_vmcnt<0>();  // this wave's loads of the next stage have landed
+          barrier();        // ... and everyone's; everyone has read the last operands of `cur`
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        acc[i][j] = mfma32(fb[ks & 1][j].template get<v8>(), fa[ks & 1][i].template get<v8>(), acc[i][j]);
+        __builtin_amdgcn_sched_barrier(0);
+        if (m >= first && (!last || MORE)) {
+#pragma unroll
+          for (int r = (m - first) * RPS; r < (m - first + 1) * RPS && r < NR; ++r) {
+            if (last) read_item(nxt, 0, 0, r);
+            else read_item(cur, ks + 1, (ks + 1) & 1, r);
+          }
+        }
+        if (m >= xfirst) {
+#pragma unroll
+          for (int q = (m - xfirst) * nx / xslots; q < (m - xfirst + 1) * nx / xslots; ++q) {
+            if (last) load_item(cur, q);                 // first half of the stage after the next one
+            else if (ks == 0) load_item(nxt, NEARLY + q);  // the rest of the next stage
+            else advance_item(q);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  };
+  typedef std::integral_constant<bool, true> yes_t;
+  typedef std::integral_constant<bool, false> no_t;
+  int kt = 0;
+  for (; kt + 2 < nk; ++kt) stage(smem + (kt & 1) * STAGE, smem + ((kt + 1) & 1) * STAGE, yes_t(), yes_t());
+  if (kt + 1 < nk) {
+    stage(smem + (kt & 1) * STAGE, smem + ((kt + 1) & 1) * STAGE, yes_t(), no_t());
+    ++kt;
+  }
+  if (kt < nk) stage(smem + (kt & 1) * STAGE, smem + ((kt + 1) & 1) * STAGE, no_t(), no_t());
 
   static_assert(NW * 32 * (WTN * 4 + 16) <= 2 * STAGE, "epilogue staging must fit in the pipeline LDS");
   if (p.splits > 1) {
