@@ -421,7 +421,7 @@ struct DmaPanel {
 // tile) instead of 32 scattered 16-byte pieces.
 // PLAIN: the caller knows that there is no bias, ReLU, mask or sign-bit work (most launches of a
 // training step): the write-out is then straight-line code without the tests for them.
-template <typename T, typename TO, int TM, int TN, int WTM, int WTN, bool PLAIN = false>
+template <typename T, typename TO, int TM, int TN, int WTM, int WTN, bool PLAIN = false, bool FULL = false>
 __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x16 (&acc)[TM][TN], char* smem, int m0,
                                                   int n0, int wm, int wn, int wave, int lane,
                                                   const uint8_t (*sign_bytes)[4] = nullptr) {
@@ -444,6 +444,8 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x16 (&
   // step of the 410M model: the store loop is where short-contraction launches spend their time)
   const int n_lane = nbase + (lane % CH) * EPC;
   const int64_t col_off = n_lane + (int64_t)(n_lane / p.chunk_n) * p.chunk_skip;
+  // ... and so is the row part of its first store; the others lie whole multiples of ldc further on
+  TO* const row0 = C + (int64_t)(m0 + wm * WTM + lane / CH) * p.ldc + col_off;
   // this lane's bias values: the same for every 32-row block, requested once ahead of the loop
   typename Vec<T>::v4 bvals[TN][4] = {};
   if (bias) {
@@ -488,12 +490,18 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x16 (&
         }
       }
     }
+    // all row segments of the block are requested from the slab before the first store: each store
+    // then waits for its own read only (a read followed at once by its store exposes the LDS
+    // latency once per store)
+    u32x4 vals[32 / RPI];
+#pragma unroll
+    for (int rr = 0; rr < 32 / RPI; ++rr) vals[rr] = lds_ld16(mine, (rr * RPI + lane / CH) * ROWB + (lane % CH) * 16);
 #pragma unroll
     for (int rr = 0; rr < 32 / RPI; ++rr) {
       const int r = rr * RPI + lane / CH, c = lane % CH;
-      u32x4 val = lds_ld16(mine, r * ROWB + c * 16);
+      u32x4 val = vals[rr];
       const int m = m0 + wm * WTM + i * 32 + r, n = nbase + c * EPC;
-      if (m < p.M && n < p.N) {
+      if (FULL || (m < p.M && n < p.N)) {
         if (mask) {  // ReLU gradient mask fused into the write-out: zero where the activation is not positive
           const T* mk = (const T*)mask + (int64_t)m * p.ldmask + n;
           if constexpr (ES == 2) {
@@ -539,7 +547,7 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x16 (&
             ((uint8_t*)sign_out)[(int64_t)m * p.ldsign + (n >> 3)] = (uint8_t)bits;
           }
         }
-        st16(C + (int64_t)m * p.ldc + col_off, val);
+        st16(row0 + (int64_t)(i * 32 + rr * RPI) * p.ldc, val);
       }
     }
   }
@@ -725,6 +733,7 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams& p, const int pid
   if (kt < nk) stage(smem + (kt & 1) * STAGE, smem + ((kt + 1) & 1) * STAGE, no_t(), no_t());
 
   static_assert(NW * 32 * (WTN * 4 + 16) <= 2 * STAGE, "epilogue staging must fit in the pipeline LDS");
+  const bool full = m0 + BM <= p.M && n0 + BN <= p.N;  // no row or column of the tile lies outside C: stores need no test
   if (p.splits > 1) {
     // fp32 partial of this contraction slice: a plain (M, N) matrix, written like an fp32 result
     GemmParams q = p;
@@ -739,15 +748,18 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams& p, const int pid
     q.chunk_n = p.N;
     q.chunk_skip = 0;
     __syncthreads();  // all waves are done reading the last pipeline stage
-    gemm_epilogue_lds<T, float, TM, TN, WTM, WTN, true>(q, acc, smem, m0, n0, wm, wn, wave, lane);
+    if (full) gemm_epilogue_lds<T, float, TM, TN, WTM, WTN, true, true>(q, acc, smem, m0, n0, wm, wn, wave, lane);
+    else gemm_epilogue_lds<T, float, TM, TN, WTM, WTN, true>(q, acc, smem, m0, n0, wm, wn, wave, lane);
   } else {
     __syncthreads();  // all waves are done reading the last pipeline stage
     const bool plain = !p.bias && !p.relu && !p.mask && !p.sign_in && !p.sign_out && !p.alpha;
     if (p.out_f32) {
-      if (plain) gemm_epilogue_lds<T, float, TM, TN, WTM, WTN, true>(p, acc, smem, m0, n0, wm, wn, wave, lane);
+      if (plain && full) gemm_epilogue_lds<T, float, TM, TN, WTM, WTN, true, true>(p, acc, smem, m0, n0, wm, wn, wave, lane);
+      else if (plain) gemm_epilogue_lds<T, float, TM, TN, WTM, WTN, true>(p, acc, smem, m0, n0, wm, wn, wave, lane);
       else gemm_epilogue_lds<T, float, TM, TN, WTM, WTN>(p, acc, smem, m0, n0, wm, wn, wave, lane);
     } else {
-      if (plain) gemm_epilogue_lds<T, T, TM, TN, WTM, WTN, true>(p, acc, smem, m0, n0, wm, wn, wave, lane);
+      if (plain && full) gemm_epilogue_lds<T, T, TM, TN, WTM, WTN, true, true>(p, acc, smem, m0, n0, wm, wn, wave, lane);
+      else if (plain) gemm_epilogue_lds<T, T, TM, TN, WTM, WTN, true>(p, acc, smem, m0, n0, wm, wn, wave, lane);
       else gemm_epilogue_lds<T, T, TM, TN, WTM, WTN>(p, acc, smem, m0, n0, wm, wn, wave, lane, sign_bytes);
     }
   }
