@@ -134,8 +134,18 @@ class GemmTimer:
     """HIP events on the current (launch) stream around every tf_gemm / tf_gemm_scaled / tf_gemm_relu_bits /
     tf_gemm_group call."""
 
-    def __init__(self):
+    def __init__(self, events=4096):
         self.records = []
+        # events made (and recorded once, which is when torch creates the HIP event) ahead of the
+        # instrumented steps: creating two per call inside them slows the host enough for the GPU
+        # to catch up in the forward pass, and a call's events then also cover the idle gap
+        self._pool = [torch.cuda.Event(enable_timing=True) for _ in range(events)]
+        for e in self._pool:
+            e.record()
+        torch.cuda.synchronize()
+
+    def _event(self):
+        return self._pool.pop() if self._pool else torch.cuda.Event(enable_timing=True)
 
     def __enter__(self):
         from tritonformer_amd import kernels
@@ -144,8 +154,7 @@ class GemmTimer:
         self._orig = kernels._gemm
 
         def timed(dtype, la, lb, m, n, k, *rest, **kw):
-            e0 = torch.cuda.Event(enable_timing=True)
-            e1 = torch.cuda.Event(enable_timing=True)
+            e0, e1 = self._event(), self._event()
             e0.record()
             self._orig(dtype, la, lb, m, n, k, *rest, **kw)
             e1.record()
@@ -154,8 +163,7 @@ class GemmTimer:
         self._orig_scaled = kernels._gemm_scaled
 
         def timed_scaled(dtype, la, lb, m, n, k, *rest):
-            e0 = torch.cuda.Event(enable_timing=True)
-            e1 = torch.cuda.Event(enable_timing=True)
+            e0, e1 = self._event(), self._event()
             e0.record()
             self._orig_scaled(dtype, la, lb, m, n, k, *rest)
             e1.record()
@@ -164,8 +172,7 @@ class GemmTimer:
         self._orig_group = kernels._gemm_group
 
         def timed_group(dtype, out_dtype, la, lb, problems, device):
-            e0 = torch.cuda.Event(enable_timing=True)
-            e1 = torch.cuda.Event(enable_timing=True)
+            e0, e1 = self._event(), self._event()
             e0.record()
             self._orig_group(dtype, out_dtype, la, lb, problems, device)
             e1.record()
@@ -175,8 +182,7 @@ class GemmTimer:
         self._orig_bits = kernels._gemm_bits
 
         def timed_bits(dtype, lb, m, n, k, *rest):
-            e0 = torch.cuda.Event(enable_timing=True)
-            e1 = torch.cuda.Event(enable_timing=True)
+            e0, e1 = self._event(), self._event()
             e0.record()
             rc = self._orig_bits(dtype, lb, m, n, k, *rest)
             e1.record()
