@@ -225,6 +225,7 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (BMODE == kDenseBias ? 2 : 3)) v
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);  // the same number as a scalar: LDS slot addresses of the tile loads stay scalar arithmetic
   const int nbh = p.B * p.nh;
   const int nqb = (p.S + 127) / 128;
   const int qblk = nqb - 1 - (int)(blockIdx.x / nbh);  // heaviest query blocks first
@@ -273,12 +274,12 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (BMODE == kDenseBias ? 2 : 3)) v
   auto load_tile = [&](int stage_off) {  // next 64 keys / values (/ bias columns) into the stage at byte offset stage_off
 #pragma unroll
     for (int j = 0; j < PT; ++j) {
-      __builtin_amdgcn_global_load_lds((gptr_void*)kp[j], (lds_void*)KT::stream_slot(smem + stage_off, wave, j), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_void*)kp[j], (lds_void*)KT::stream_slot(smem + stage_off, wave_u, j), 16, 0, 0);
       __builtin_amdgcn_global_load_lds((gptr_void*)(kp[j] + v_minus_k),
-                                       (lds_void*)KT::stream_slot(smem + stage_off + KT::BYTES, wave, j), 16, 0, 0);
+                                       (lds_void*)KT::stream_slot(smem + stage_off + KT::BYTES, wave_u, j), 16, 0, 0);
       kp[j] += (int64_t)64 * p.ss;
     }
-    if (HAS_BIAS) BiasTile::load(bp, smem + stage_off + 2 * KT::BYTES, wave);
+    if (HAS_BIAS) BiasTile::load(bp, smem + stage_off + 2 * KT::BYTES, wave_u);
   };
   uint32_t ka[KS], va[DT][2];
   const uint32_t lds0 = lds_address(smem);
@@ -438,6 +439,7 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_dkdv_kernel(AttnPa
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);  // the same number as a scalar: LDS slot addresses of the tile loads stay scalar arithmetic
   const int nbh = p.B * p.nh;
   const int kblk = (int)(blockIdx.x / nbh);  // lowest key blocks (longest loops) first
   const int bh = blockIdx.x % nbh;
@@ -495,20 +497,20 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_dkdv_kernel(AttnPa
   auto load_block = [&](int stage_off) {  // next 64 queries into the stage at byte offset stage_off
 #pragma unroll
     for (int j = 0; j < PT; ++j) {
-      __builtin_amdgcn_global_load_lds((gptr_void*)qp[j], (lds_void*)QT::stream_slot(smem + stage_off, wave, j), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((gptr_void*)dop[j], (lds_void*)QT::stream_slot(smem + stage_off + QT::BYTES, wave, j),
+      __builtin_amdgcn_global_load_lds((gptr_void*)qp[j], (lds_void*)QT::stream_slot(smem + stage_off, wave_u, j), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_void*)dop[j], (lds_void*)QT::stream_slot(smem + stage_off + QT::BYTES, wave_u, j),
                                        16, 0, 0);
       qp[j] += (int64_t)64 * p.ss;
       dop[j] += (int64_t)64 * p.oss;
     }
     if (wave < 2) {
-      __builtin_amdgcn_global_load_lds((gptr_void*)statp, (lds_void*)(smem + stage_off + STAT + wave * 256), 4, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_void*)statp, (lds_void*)(smem + stage_off + STAT + wave_u * 256), 4, 0, 0);
       statp += 64;
     }
     if (HAS_BIAS) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        __builtin_amdgcn_global_load_lds((gptr_void*)bp[j], (lds_void*)(smem + stage_off + BIAS + (j * 256 + wave * 64) * 16),
+        __builtin_amdgcn_global_load_lds((gptr_void*)bp[j], (lds_void*)(smem + stage_off + BIAS + (j * 256 + wave_u * 64) * 16),
                                          16, 0, 0);
         bp[j] += (int64_t)64 * p.bias_sr;
       }
@@ -659,6 +661,7 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (BMODE != kNoBias ? 2 : 3)) void
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);  // the same number as a scalar: LDS slot addresses of the tile loads stay scalar arithmetic
   const int nbh = p.B * p.nh;
   const int nqb = (p.S + 127) / 128;
   const int qblk = nqb - 1 - (int)(blockIdx.x / nbh);
@@ -724,12 +727,12 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (BMODE != kNoBias ? 2 : 3)) void
   auto load_tile = [&](int stage_off) {
 #pragma unroll
     for (int j = 0; j < PT; ++j) {
-      __builtin_amdgcn_global_load_lds((gptr_void*)kp[j], (lds_void*)KT::stream_slot(smem + stage_off, wave, j), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_void*)kp[j], (lds_void*)KT::stream_slot(smem + stage_off, wave_u, j), 16, 0, 0);
       __builtin_amdgcn_global_load_lds((gptr_void*)(kp[j] + v_minus_k),
-                                       (lds_void*)KT::stream_slot(smem + stage_off + KT::BYTES, wave, j), 16, 0, 0);
+                                       (lds_void*)KT::stream_slot(smem + stage_off + KT::BYTES, wave_u, j), 16, 0, 0);
       kp[j] += (int64_t)64 * p.ss;
     }
-    if (HAS_BIAS) BiasTile::load(bp, smem + stage_off + 2 * KT::BYTES, wave);
+    if (HAS_BIAS) BiasTile::load(bp, smem + stage_off + 2 * KT::BYTES, wave_u);
   };
   // row operands of K and V, hd operands of K
   uint32_t ra[KS], ha[DT][2];
