@@ -30,6 +30,10 @@ __global__ __launch_bounds__(256) void ln_fwd_vec(int64_t rows, int d, const T* 
   // beside the reductions and the stores of the row before: with one row per wave and every wave
   // of the launch resident at once, the whole launch reads first and writes afterwards, and
   // neither half of the memory system's time is used by the other.
+  // The add + LayerNorm instantiation must give the bits of an addition followed by the plain one:
+  // no contraction left to the compiler (it may fuse differently per instantiation), the fused
+  // operations are spelled out.
+#pragma clang fp contract(off)
   const int lane = threadIdx.x & 63;
   const int nchunk = d >> 3;
   const int64_t stride = (int64_t)gridDim.x * kRowsPerBlock;
@@ -46,6 +50,18 @@ __global__ __launch_bounds__(256) void ln_fwd_vec(int64_t rows, int d, const T* 
   };
   int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
   if (row < rows) fetch(row);
+  // this lane's gamma and beta are the same for every row it walks: held in registers (inside the
+  // row loop they would be fetched again per row -- the stores keep the compiler from hoisting them --
+  // and at d = 1024 with fp32 parameters that is twice the bytes of the row itself through the L1)
+  float g[NV][8], b[NV][8];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = lane + i * 64;
+    if (c < nchunk) {
+      load8<TP>(gamma + c * 8, g[i]);
+      load8<TP>(beta + c * 8, b[i]);
+    }
+  }
   for (; row < rows; row += stride) {
     float v[NV][8];
     float s = 0.f;
@@ -77,7 +93,7 @@ __global__ __launch_bounds__(256) void ln_fwd_vec(int64_t rows, int d, const T* 
     for (int i = 0; i < NV; ++i) {
       if (lane + i * 64 < nchunk) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) { const float t = v[i][e] - mean; q += t * t; }
+        for (int e = 0; e < 8; ++e) { const float t = v[i][e] - mean; q = __builtin_fmaf(t, t, q); }
       }
     }
     const float var = wave_sum(q) / (float)d;
@@ -88,11 +104,15 @@ __global__ __launch_bounds__(256) void ln_fwd_vec(int64_t rows, int d, const T* 
     for (int i = 0; i < NV; ++i) {
       const int c = lane + i * 64;
       if (c < nchunk) {
-        float g[8], b[8], o[8];
-        load8<TP>(gamma + c * 8, g);
-        load8<TP>(beta + c * 8, b);
+        float o[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) o[e] = (v[i][e] - mean) * rstd * g[e] + b[e];
+        for (int e = 0; e < 8; ++e) {
+          o[e] = __builtin_fmaf((v[i][e] - mean) * rstd, g[i][e], b[i][e]);
+          // the fp32 value is pinned before the rounding to 16 bits: left alone, the compiler turns
+          // some of these into v_fma_mix*_f16 (one rounding straight to 16 bits) and others not,
+          // differently per instantiation, and the two forms differ in one element in 50 000
+          asm("" : "+v"(o[e]));
+        }
         Chunk<T>::store(yr + c * 8, o);
       }
     }
@@ -127,7 +147,7 @@ __global__ __launch_bounds__(256) void ln_fwd_any(int64_t rows, int d, const T* 
   if (lane == 0) { mean_out[row] = mean; rstd_out[row] = rstd; }
   T* yr = y + row * ldy;
   for (int c = lane; c < d; c += 64)
-    yr[c] = (T)(((float)xr[c] - mean) * rstd * (float)gamma[c] + (float)beta[c]);
+    yr[c] = (T)__builtin_fmaf(((float)xr[c] - mean) * rstd, (float)gamma[c], (float)beta[c]);
 }
 
 // ---------------------------------------------------------------------------
