@@ -640,16 +640,20 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams& p, const int pid
     PB::issue(pb, smem + PA::BYTES, wave);
     PA::advance(pa, p.lda);
     PB::advance(pb, p.ldb);
-    wait_vmcnt<0>();
-    barrier();
-    read_operands(smem, 0, 0);
+    // the head of step 1 goes out before step 0 is waited for: the two travel together through
+    // the cold start instead of one after the other
     if (nk > 1) {
 #pragma unroll
       for (int q = 0; q < NEARLY; ++q) {
         if (q < PA::PER_WAVE) PA::issue_one(pa, smem + STAGE, wave, q);
         else PB::issue_one(pb, smem + STAGE + PA::BYTES, wave, q - PA::PER_WAVE);
       }
+      wait_vmcnt<NEARLY>();  // loads complete in order: all but the NEARLY youngest = step 0
+    } else {
+      wait_vmcnt<0>();
     }
+    barrier();
+    read_operands(smem, 0, 0);
   }
 
   // ---- main loop.  Every LDS read, load and pointer update sits behind an MFMA, pinned there by
