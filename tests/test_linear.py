@@ -283,6 +283,33 @@ def test_every_tile_configuration_gives_the_same_product(layouts, dev):
         assert rel_l2(run(cfg, 4, 0), base) < 1e-3, f"cfg {cfg} split 4"
 
 
+@pytest.mark.parametrize("layouts", ["fwd", "dx", "dw"])
+def test_short_contractions_take_every_peeled_form_of_the_main_loop(layouts, dev):
+    """One, two, three, four and five 64-wide stages: the main loop of the direct-to-LDS kernels peels
+    its last two stages (no stage after, one stage after) from the steady state, and its prologue
+    requests the head of the second stage before it waits for the first.  Every tile configuration,
+    against fp32 math, with and without a split that leaves a single stage per slice."""
+    from tritonformer_amd import _lib
+
+    d = _lib.load_diag()
+    g = torch.Generator().manual_seed(31)
+    M, N = 384, 512
+    la, lb = {"fwd": (0, 1), "dx": (0, 0), "dw": (1, 1)}[layouts]
+    stream = torch.cuda.current_stream().cuda_stream
+    for K in (64, 128, 192, 256, 320):
+        a = torch.randn((M, K) if la == 0 else (K, M), generator=g).half().to(dev)
+        b = (torch.randn((N, K) if lb == 0 else (K, N), generator=g) / K ** 0.5).half().to(dev)
+        want = (a.float() if la == 0 else a.float().T) @ (b.float().T if lb == 0 else b.float())
+        for cfg in range(2, 6):
+            for splits in (1, K // 64):
+                out = torch.empty((M, N), dtype=torch.float16, device=dev)
+                nb = d.tf_diag_gemm_workspace_bytes(cfg, splits, M, N, K)
+                ws = torch.empty(max(nb, 16), dtype=torch.uint8, device=dev)
+                _lib.check(d.tf_diag_gemm(stream, cfg, splits, 0, 0, 0, la, lb, M, N, K, a.data_ptr(), a.stride(0),
+                                          b.data_ptr(), b.stride(0), out.data_ptr(), N, None, 0, ws.data_ptr(), nb))
+                assert_close(out, want, name=f"{layouts} K={K} cfg {cfg} splits {splits}")
+
+
 @pytest.mark.parametrize("dims,use_bias", [((2, 128, 256, 1024), False), ((3, 77, 136, 264), True),
                                            ((1, 100, 333, 129), True)])
 def test_fused_mlp_equals_two_functions(dims, use_bias, dev):
