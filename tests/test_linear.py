@@ -283,28 +283,6 @@ def test_every_tile_configuration_gives_the_same_product(layouts, dev):
         assert rel_l2(run(cfg, 4, 0), base) < 1e-3, f"cfg {cfg} split 4"
 
 
-def test_grouped_weight_gradients_on_unsplit_small_tiles(dev):
-    """Two weight gradients whose 256x256 tiles would need a split contraction while their 128x128
-    tiles fill one round of two workgroups per CU (the MLP pair of the 410M model, here over 2048
-    tokens) run unsplit on the small tiles: against fp32 math, and against the two products launched
-    one by one (same 16-bit operands, fp32 sums in another order)."""
-    from tritonformer_amd.kernels import mm_dw, mm_dw_group
-
-    g = torch.Generator().manual_seed(41)
-    x = torch.randn(1, 2048, 1024, generator=g).half().to(dev)
-    h = torch.randn(1, 2048, 4096, generator=g).half().to(dev)
-    dy = torch.randn(1, 2048, 1024, generator=g).half().to(dev)
-    dh = torch.randn(1, 2048, 4096, generator=g).half().to(dev)
-    dw1, dw2 = mm_dw_group([(x, dh), (h, dy)], out_dtype=torch.float32)
-    assert dw1.shape == (1024, 4096) and dw2.shape == (4096, 1024) and dw1.dtype == torch.float32
-    for got, a, b in ((dw1, x, dh), (dw2, h, dy)):
-        want = a[0].float().T @ b[0].float()
-        assert rel_l2(got, want) < 1e-5
-        assert rel_l2(got, mm_dw(a, b, out_dtype=torch.float32)) < 1e-5
-    lo1, lo2 = mm_dw_group([(x, dh), (h, dy)])      # 16-bit results take the same path
-    assert lo1.dtype == torch.float16 and rel_l2(lo1, dw1) < 1e-3 and rel_l2(lo2, dw2) < 1e-3
-
-
 @pytest.mark.parametrize("layouts", ["fwd", "dx", "dw"])
 def test_short_contractions_take_every_peeled_form_of_the_main_loop(layouts, dev):
     """One, two, three, four and five 64-wide stages: the main loop of the direct-to-LDS kernels peels

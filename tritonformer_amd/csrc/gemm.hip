@@ -1068,20 +1068,12 @@ static int gemm_dispatch(hipStream_t st, int la, int lb, bool vec, const GemmPla
 // One launch for a group of weight-gradient style products (both operands contraction-strided),
 // 256x256 tiles, direct-to-LDS kernel; then one reduce pass per problem.
 template <typename T>
-static int gemm_group_dispatch(hipStream_t st, const GemmGroup& g, int tile) {
-  if (tile == 128) {
-    constexpr int lds = 2 * (128 + 128) * 64 * 2;
-    auto kernel = gemm_dma_group_kernel<T, 128, 128, 64, 2, 2, 2, false, false>;
-    static bool once = (allow_big_lds(kernel, lds), true);
-    (void)once;
-    kernel<<<dim3((unsigned)g.first[g.count]), dim3(256), lds, st>>>(g);
-  } else {
-    constexpr int lds = 2 * (256 + 256) * 64 * 2;
-    auto kernel = gemm_dma_group_kernel<T, 256, 256, 64, 2, 4, 2, false, false>;
-    static bool once = (allow_big_lds(kernel, lds), true);
-    (void)once;
-    kernel<<<dim3((unsigned)g.first[g.count]), dim3(512), lds, st>>>(g);
-  }
+static int gemm_group_dispatch(hipStream_t st, const GemmGroup& g) {
+  constexpr int lds = 2 * (256 + 256) * 64 * 2;
+  auto kernel = gemm_dma_group_kernel<T, 256, 256, 64, 2, 4, 2, false, false>;
+  static bool once = (allow_big_lds(kernel, lds), true);
+  (void)once;
+  kernel<<<dim3((unsigned)g.first[g.count]), dim3(512), lds, st>>>(g);
   TF_CHECK_LAUNCH();
   g_gemm_launches.fetch_add(1, std::memory_order_relaxed);
   // second pass of the split contractions: all products of the group in one launch
@@ -1344,7 +1336,6 @@ struct GroupPlan {
   bool grouped;   // one launch for all problems (otherwise: one tf_gemm_out_chunked call each)
   int splits;
   int64_t need;   // workspace bytes
-  int tile;       // 256 or 128: edge of the square tiles
 };
 
 bool group_problem_ok(const tf_gemm_problem& q) {
@@ -1361,15 +1352,14 @@ bool group_problem_fast(const tf_gemm_problem& q) {
 }
 
 GroupPlan plan_group(int la, int lb, int count, const tf_gemm_problem* pr) {
-  GroupPlan gp = {false, 1, 0, 256};
+  GroupPlan gp = {false, 1, 0};
   bool fast = count >= 2 && count <= kMaxGroup && la == TF_OP_KMINOR && lb == TF_OP_KMINOR;
   const int64_t cus = device_shape().cus;
-  int64_t tiles = 0, tiles128 = 0, min_ksteps = INT64_MAX;
+  int64_t tiles = 0, min_ksteps = INT64_MAX;
   for (int i = 0; i < count && fast; ++i) {
     fast = group_problem_ok(pr[i]) && group_problem_fast(pr[i]);
     if (!fast) break;
     tiles += ((pr[i].M + 255) / 256) * ((pr[i].N + 255) / 256);
-    tiles128 += ((pr[i].M + 127) / 128) * ((pr[i].N + 127) / 128);
     const int64_t ks = pr[i].K / 64;
     if (ks < min_ksteps) min_ksteps = ks;
   }
@@ -1382,14 +1372,6 @@ GroupPlan plan_group(int la, int lb, int count, const tf_gemm_problem* pr) {
       const int64_t max_by_k = min_ksteps / 16 > 0 ? min_ksteps / 16 : 1;
       if (splits > max_by_k) splits = max_by_k;
       if (splits > 16) splits = 16;
-    }
-    // Where 256x256 tiles would have to split the contraction but 128x128 tiles fill one round of two
-    // workgroups per CU, the smaller tiles go unsplit: no fp32 partials (64 MiB written and read again
-    // per launch for the two MLP weight gradients of the 410M model) and no reduce pass, at the same
-    // GEMM time; -0.1 ms per step.  With one workgroup per CU or less the smaller tiles lose.
-    if (splits > 1 && tiles128 > cus && tiles128 <= 2 * cus) {
-      gp.tile = 128;
-      splits = 1;
     }
     gp.grouped = true;
     gp.splits = (int)splits;
@@ -1442,7 +1424,7 @@ extern "C" int tf_gemm_group(void* stream, int dtype, int out_dtype, int layout_
     p.M = (int)q.M; p.N = (int)q.N; p.K = (int)q.K;
     p.lda = q.lda; p.ldb = q.ldb; p.ldc = q.ldc;
     p.relu = 0;
-    p.tiles_m = (int)((q.M + gp.tile - 1) / gp.tile); p.tiles_n = (int)((q.N + gp.tile - 1) / gp.tile);
+    p.tiles_m = (int)((q.M + 255) / 256); p.tiles_n = (int)((q.N + 255) / 256);
     const int64_t ksteps = q.K / 64;
     const int64_t steps_per = (ksteps + gp.splits - 1) / gp.splits;
     p.k_per_split = (int)(steps_per * 64);
@@ -1461,6 +1443,6 @@ extern "C" int tf_gemm_group(void* stream, int dtype, int out_dtype, int layout_
     }
   }
   hipStream_t st = (hipStream_t)stream;
-  if (dtype == TF_F16) return gemm_group_dispatch<f16>(st, g, gp.tile);
-  return gemm_group_dispatch<bf16>(st, g, gp.tile);
+  if (dtype == TF_F16) return gemm_group_dispatch<f16>(st, g);
+  return gemm_group_dispatch<bf16>(st, g);
 }
