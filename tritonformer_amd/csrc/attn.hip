@@ -121,15 +121,23 @@ __device__ __forceinline__ float max_with_other_half(float x) {
 // Bias modes of the kernels: none, a dense (nh, S', S') matrix, ALiBi in closed form.
 constexpr int kNoBias = 0, kDenseBias = 1, kAlibi = 2;
 
-// ALiBi bias of one (query, key) pair times log2(e), bit for bit what the dense path reads from
-// the matrix the reference builds (transformer.py:55-75): the distance key - query (<= 0) and the
-// slope are fp16 values, their product is rounded to fp16 once, a bf16 kernel sees that value
-// rounded to bf16 (the 16-bit matrix cast to the compute type).
-template <typename T> __device__ __forceinline__ float alibi_log2(float dist, _Float16 slope) {
-  const _Float16 b16 = (_Float16)dist * slope;
-  float b = (float)b16;
-  if (std::is_same<T, bf16>::value) b = (float)(T)b;
-  return b * kLog2e;
+// ALiBi biases of four consecutive (query, key) distances d0, d0 + step, ..., bit for bit what the dense
+// path reads from the matrix the reference builds (transformer.py:55-75): the distance key - query
+// (<= 0) and the slope are fp16 values, their product is rounded to fp16 once, a bf16 kernel sees that
+// value rounded to bf16 (the 16-bit matrix cast to the compute type).  Two distances are rounded to fp16
+// by one conversion and multiplied by one packed fp16 instruction.  Returned as floats, NOT yet
+// multiplied by log2(e): that product rides in the fma that adds the bias to the scaled score.
+template <typename T> __device__ __forceinline__ void alibi4(float d0, float step, _Float16 slope, float (&b)[4]) {
+  typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+  typedef float f2 __attribute__((ext_vector_type(2)));
+  const f2 da = {d0, d0 + step}, db = {d0 + 2.f * step, d0 + 3.f * step};
+  const h2 s2 = {slope, slope};
+  const h2 pa = __builtin_convertvector(da, h2) * s2, pb = __builtin_convertvector(db, h2) * s2;
+  b[0] = (float)pa[0]; b[1] = (float)pa[1]; b[2] = (float)pb[0]; b[3] = (float)pb[1];
+  if (std::is_same<T, bf16>::value) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) b[e] = (float)(T)b[e];
+  }
 }
 
 // Additive-bias tile of a 128-query block and a 64-key block, 16 KB, staged through LDS with
@@ -337,17 +345,14 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (BMODE == kDenseBias ? 2 : 3)) v
               lds_wait<7 - decltype(it)::value>(braw[jt * 4 + g]);
               const v4 raw = __builtin_bit_cast(v4, braw[jt * 4 + g]);
 #pragma unroll
-              for (int e = 0; e < 4; ++e) bv[e] = (float)raw[e] * kLog2e;
+              for (int e = 0; e < 4; ++e) bv[e] = (float)raw[e];
             }
-            if constexpr (ALIBI) {
-              const float d0 = (float)(key0 - myq);
-#pragma unroll
-              for (int e = 0; e < 4; ++e) bv[e] = alibi_log2<T>(d0 + (float)e, slope);
-            }
+            if constexpr (ALIBI) alibi4<T>((float)(key0 - myq), 1.f, slope, bv);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               float x = st[jt][g * 4 + e];
-              if (HAS_BIAS || ALIBI) x = fmaf(x, p.scale_log2, bv[e]);
+              // score * scale * log2e + bias * log2e: the 16-bit bias goes into the fma as it is
+              if (HAS_BIAS || ALIBI) x = __builtin_fmaf(bv[e], kLog2e, x * p.scale_log2);
               if (DIAG && (key0 + e > myq || (jt == 1 && !live1))) x = -INFINITY;
               st[jt][g * 4 + e] = x;
               mx = fmaxf(mx, x);
@@ -596,12 +601,14 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_dkdv_kernel(AttnPa
             constexpr int g = decltype(gt)::value;
             const int ql = qt * 32 + g * 8 + 4 * (lane >> 5);  // block-local first query of the group
             const f32x4 l4 = __builtin_bit_cast(f32x4, ls[g]);
+            float bv[4] = {0.f, 0.f, 0.f, 0.f};
+            if constexpr (ALIBI) alibi4<T>((float)(mykey - (qb + ql)), -1.f, slope, bv);  // queries ascend: distances descend
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               const int qi = qb + ql + e;
               float x = fmaf(s[g * 4 + e], p.scale_log2, -l4[e]);  // s*scale*log2e - lse
-              if constexpr (HAS_BIAS) x += (float)__builtin_bit_cast(T, (uint16_t)braw[g * 4 + e]) * kLog2e;
-              if constexpr (ALIBI) x += alibi_log2<T>((float)(mykey - qi), slope);
+              if constexpr (HAS_BIAS) bv[e] = (float)__builtin_bit_cast(T, (uint16_t)braw[g * 4 + e]);
+              if constexpr (HAS_BIAS || ALIBI) x = __builtin_fmaf(bv[e], kLog2e, x);
               float pr = fast_exp2(x);
               if (DIAG && mykey > qi) pr = 0.f;
               s[g * 4 + e] = pr;
@@ -801,17 +808,13 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (BMODE != kNoBias ? 2 : 3)) void
               lds_wait<(later < 15 ? later : 15)>(braw[g]);
               const v4 raw = __builtin_bit_cast(v4, braw[g]);
 #pragma unroll
-              for (int e = 0; e < 4; ++e) bv[e] = (float)raw[e] * kLog2e;
+              for (int e = 0; e < 4; ++e) bv[e] = (float)raw[e];
             }
-            if constexpr (ALIBI) {
-              const float d0 = (float)(key0 - myq);
-#pragma unroll
-              for (int e = 0; e < 4; ++e) bv[e] = alibi_log2<T>(d0 + (float)e, slope);
-            }
+            if constexpr (ALIBI) alibi4<T>((float)(key0 - myq), 1.f, slope, bv);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               float x = fmaf(s[g * 4 + e], p.scale_log2, neg_lse);
-              if (HAS_BIAS || ALIBI) x += bv[e];
+              if (HAS_BIAS || ALIBI) x = __builtin_fmaf(bv[e], kLog2e, x);
               float pr = fast_exp2(x);
               if (DIAG && key0 + e > myq) pr = 0.f;
               dp[g * 4 + e] *= pr;
