@@ -15,11 +15,15 @@ value        = algorithmic FLOPs of the step (6*T*P_mat + 7*L*B*S^2*d) / step ti
 extras       = the same step timed in the other regimes, in the same run: `loss_scaled` (backward of
                loss * 1024: without scaling, fp16 flushes most of the 1/N-scaled logit gradients to
                zero and the backward GEMMs multiply near-constant operands, which the matrix cores run
-               at a higher clock), `recast_each_step` (weights converted in every forward pass), and
-               `workloads` (the other configurations of the baseline)
+               at a higher clock), `recast_each_step` (weights converted in every forward pass),
+               `training_regime` (both of these at once: what a step followed by an optimizer pays),
+               `drop_in_graph` (every model-level fusion off: the reference's graph node for node through
+               the reference-named Functions) and `workloads` (the other configurations of the baseline)
 roofline     = the GEMM kernel (dominant in time): algorithmic FLOPs per launch / mean launch
                duration, the duration measured with HIP events recorded on the launch stream
-               around every GEMM launch in instrumented repeats of the same steps
+               around every GEMM launch in instrumented repeats of the same steps; `other_kernels`
+               holds the same for the attention kernels (against MFMA peak) and for the LayerNorm and
+               cross-entropy kernels (algorithmic bytes against HBM peak)
 cpu_baseline = the fp32 PyTorch oracle (oracle/ref_torch.py) on the host cores, on a bounded
                sample: the same step with the stack cut to 2 layers
 """
@@ -130,11 +134,51 @@ def gemm_table(by_shape, reps, workload, dtype_name):
     return "\n".join(head + [r[1] for r in rows]) + "\n"
 
 
+def _attn_flop(fwd):
+    # args: stream, dtype, B, nh, S, hd, ...; causal: 2 (forward) or 5 (backward) products at half cost
+    return lambda a: (2.0 if fwd else 5.0) * a[2] * a[3] * a[4] * a[4] * a[5]
+
+
+# C-ABI entry point -> (kernel family, algorithmic FLOPs or HBM bytes of one call).  Bytes: every operand
+# and result of the call once, 2 bytes per element (fp32 statistics and parameter vectors left out):
+# LayerNorm forward reads x, writes y; its backward reads dy, x, writes dx; the residual forms read and
+# write one more stream each; cross-entropy forward + gradient reads the logits and writes their gradient.
+FAMILY_ENTRY_POINTS = {
+    "tf_attn_fwd": ("attention", _attn_flop(True)),
+    "tf_attn_bwd": ("attention", _attn_flop(False)),
+    "tf_attn_alibi_fwd": ("attention", _attn_flop(True)),
+    "tf_attn_alibi_bwd": ("attention", _attn_flop(False)),
+    "tf_layernorm_fwd": ("layernorm", lambda a: 4.0 * a[3] * a[4]),
+    "tf_layernorm_bwd": ("layernorm", lambda a: 6.0 * a[3] * a[4]),
+    "tf_add_layernorm_fwd": ("layernorm", lambda a: 8.0 * a[3] * a[4]),
+    "tf_add_layernorm_bwd": ("layernorm", lambda a: 8.0 * a[3] * a[4]),
+    "tf_cross_entropy_fwd": ("cross_entropy", lambda a: 2.0 * a[2] * a[3]),
+    "tf_cross_entropy_fwd_grad": ("cross_entropy", lambda a: 4.0 * a[2] * a[3]),
+    "tf_cross_entropy_bwd": ("cross_entropy", lambda a: 4.0 * a[2] * a[3]),
+}
+FAMILY_BOUND = {"attention": ("mfma", PEAK_FP16_TFLOPS, "TFLOP/s", 1e12),
+                "layernorm": ("hbm", PEAK_HBM_GBS, "GB/s", 1e9),
+                "cross_entropy": ("hbm", PEAK_HBM_GBS, "GB/s", 1e9)}
+
+
+def family_rooflines(by_family, reps):
+    """One roofline block per kernel family, from the events of the instrumented steps."""
+    out = []
+    for family, (cnt, ms, work) in sorted(by_family.items()):
+        bound, peak, unit, per = FAMILY_BOUND[family]
+        achieved = work / (ms * 1e-3) / per
+        out.append({"family": family, "bound": bound, "achieved": round(achieved, 1), "peak": peak, "unit": unit,
+                    "frac": round(achieved / peak, 4), "calls_per_step": cnt // reps,
+                    "avg_call_us": round(ms / cnt * 1e3, 2), "ms_per_step": round(ms / reps, 3),
+                    "work_per_call": round(work / cnt, 1)})
+    return out
+
+
 class GemmTimer:
     """HIP events on the current (launch) stream around every tf_gemm / tf_gemm_scaled / tf_gemm_relu_bits /
-    tf_gemm_group call."""
+    tf_gemm_group call, and around every attention, LayerNorm and cross-entropy call (`by_family`)."""
 
-    def __init__(self, events=4096):
+    def __init__(self, events=8192):
         self.records = []
         # events made (and recorded once, which is when torch creates the HIP event) ahead of the
         # instrumented steps: creating two per call inside them slows the host enough for the GPU
@@ -194,6 +238,26 @@ class GemmTimer:
         kernels._gemm_scaled = timed_scaled
         kernels._gemm_group = timed_group
         kernels._gemm_bits = timed_bits
+
+        # the other kernel families: events around the C-ABI call itself (the launchers look the entry
+        # point up on the library object at every call, so replacing the attribute is enough)
+        self._lib = kernels.load()
+        self._lib_orig = {}
+        self.family_records = []
+        for name, (family, work) in FAMILY_ENTRY_POINTS.items():
+            orig = getattr(self._lib, name)
+            self._lib_orig[name] = orig
+
+            def timed_entry(*args, _orig=orig, _family=family, _work=work):
+                e0, e1 = self._event(), self._event()
+                e0.record()
+                rc = _orig(*args)
+                e1.record()
+                if rc == 0:
+                    self.family_records.append((_family, _work(args), e0, e1))
+                return rc
+
+            setattr(self._lib, name, timed_entry)
         return self
 
     def __exit__(self, *exc):
@@ -201,7 +265,13 @@ class GemmTimer:
         self._kernels._gemm_scaled = self._orig_scaled
         self._kernels._gemm_group = self._orig_group
         self._kernels._gemm_bits = self._orig_bits
+        for name, orig in self._lib_orig.items():
+            setattr(self._lib, name, orig)
         torch.cuda.synchronize()
+        self.by_family = {}
+        for family, work, e0, e1 in self.family_records:
+            cnt, tot, w = self.by_family.get(family, (0, 0.0, 0.0))
+            self.by_family[family] = (cnt + 1, tot + e0.elapsed_time(e1), w + work)
         self.by_shape = {}
         for key, e0, e1 in self.records:
             ms = e0.elapsed_time(e1)
@@ -475,6 +545,11 @@ def main():
                         "run after the timed ones; the event time of a call covers its GEMM kernel(s) and, for a split contraction, "
                         "the reduce kernel; launches = GEMM kernels counted by the library",
         }
+        out["roofline"]["other_kernels"] = family_rooflines(gt.by_family, reps)
+        out["roofline"]["other_kernels_measured"] = (
+            "same instrumented steps: HIP events around every tf_attn_* / tf_*layernorm_* / tf_cross_entropy_* call; "
+            "attention: 2 (forward) + 5 (backward) causal tile products; LayerNorm and cross-entropy: operand and result "
+            "bytes of the call, each once, against 8 TB/s")
         if args.gemm_table:
             with open(args.gemm_table, "w") as fh:
                 fh.write(gemm_table(gt.by_shape, reps, args.workload, args.dtype))
@@ -486,9 +561,34 @@ def main():
         if not args.recast:
             T.set_weight_cast_cache(False)
             ms_r, _ = time_steps(model, tokens, k, w, dtype)
-            T.set_weight_cast_cache(True)
             out["recast_each_step"] = {"ms_per_step": round(ms_r, 3), "steps": k,
                                        "value": round(flops / (ms_r * 1e-3) / 1e12, 2)}
+            # what a real training step pays, both at once: loss scaled (real data in the backward GEMMs)
+            # AND the fp32 weights converted in every forward pass (an optimizer changes them every step)
+            ms_t, loss_t = time_steps(model, tokens, k, w, dtype, loss_scale=args.loss_scale)
+            out["training_regime"] = {"loss_scale": args.loss_scale, "weight_casts": "every forward pass",
+                                      "ms_per_step": round(ms_t, 3), "steps": k,
+                                      "value": round(flops / (ms_t * 1e-3) / 1e12, 2),
+                                      "pct_of_fp16_mfma_peak": round(100.0 * flops / (ms_t * 1e-3) / 1e12 / PEAK_FP16_TFLOPS, 2),
+                                      "loss": round(loss_t, 4)}
+            T.set_weight_cast_cache(True)
+        # the reference's graph node for node: every model-level fusion off, so that the step runs through the
+        # reference-named Functions only (LinearNoBias x 4 + LinearNoBiasReLU per block, CausalAttention,
+        # LayerNorm, `residual + hidden`, nn.Embedding, logits + CrossEntropyLoss); headline protocol otherwise
+        import tritonformer_amd.transformer as TM
+        flags = ("FUSE_QKV", "FUSE_MLP", "FUSE_ATTN_BLOCK", "FUSE_ADD_LN", "FUSE_EMBED", "FUSE_HEAD")
+        saved = {n: getattr(TM, n) for n in flags}
+        try:
+            for n in flags:
+                setattr(TM, n, False)
+            ms_d, loss_d = time_steps(model, tokens, k, w, dtype)
+        finally:
+            for n, v in saved.items():
+                setattr(TM, n, v)
+        out["drop_in_graph"] = {"fusions": "all off (" + ", ".join(flags) + ")", "ms_per_step": round(ms_d, 3), "steps": k,
+                                "value": round(flops / (ms_d * 1e-3) / 1e12, 2),
+                                "pct_of_fp16_mfma_peak": round(100.0 * flops / (ms_d * 1e-3) / 1e12 / PEAK_FP16_TFLOPS, 2),
+                                "loss": round(loss_d, 4)}
         del model
         others = []
         for name, dts in (("gpt2-160m-ctx2048-bs8", ["fp16"]), ("gpt2-410m-ctx2048-bs4", ["fp16"]),

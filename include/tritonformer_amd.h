@@ -10,8 +10,11 @@
  * Conventions
  *  - every pointer is a DEVICE pointer unless said otherwise; the library
  *    never allocates, frees, retains or synchronises; it reads no environment
- *    variable and keeps no state between calls beyond the device's CU / XCD
- *    counts; work is enqueued on
+ *    variable.  What it keeps between calls: the device's CU / XCD counts (read
+ *    from the runtime once per device), the address of the scratch array of
+ *    tf_colsum_noalloc (taken once per device), and a counter of GEMM launches
+ *    (a relaxed atomic that only tf_diag_gemm_launch_count reads); no result
+ *    depends on any of them beyond tile choice.  Work is enqueued on
  *    `stream` (a hipStream_t passed as void*, NULL = the null stream);
  *  - strides and leading dimensions are in ELEMENTS, sizes in elements;
  *  - `dtype`: TF_F16 / TF_BF16 for the 16-bit paths, TF_F32 only where stated;
@@ -116,10 +119,11 @@ int tf_gemm_out_chunked(void* stream, int dtype, int out_dtype, int layout_a, in
  *             (the forward of LinearNoBiasReLU / LinearBiasReLU, tritonformer/linear.py:47-102);
  *   bits_in:  C = bit ? A . B : 0, no bias (mask_grad of kernels/activation.py:27-44
  *             fused into dH = dY . W2^T, reading a sixteenth of what the activation holds).
- * Served by the write-out of the direct-to-LDS kernels only: returns TF_EINVAL when
- * their preconditions (16-byte aligned operands, extents and leading dimensions
- * multiples of 8, K a multiple of 64) do not hold; callers then use tf_gemm_out with
- * the activation as mask_act.  Needs no workspace. */
+ * Served by the write-out of the direct-to-LDS kernels only: returns TF_ESHAPE (and
+ * launches nothing) when their preconditions (16-byte aligned operands, extents and
+ * leading dimensions multiples of 8, K a multiple of 64, a product large enough to run
+ * unsplit) do not hold; callers then use tf_gemm_out with the activation as mask_act.
+ * Malformed calls get the other codes as everywhere.  Needs no workspace. */
 int tf_gemm_relu_bits(void* stream, int dtype, int out_dtype, int layout_a, int layout_b,
                       int64_t M, int64_t N, int64_t K,
                       const void* A, int64_t lda, const void* B, int64_t ldb,

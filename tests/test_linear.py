@@ -13,6 +13,7 @@ import pytest
 import torch
 
 import tritonformer_amd as T
+import tritonformer_amd.kernels as K_mod
 from oracle import ref_torch as R
 from tests.util import NUM_TEST, assert_close, rel_l2
 
@@ -503,3 +504,33 @@ def test_product_cut_into_whole_rounds_and_remainder(dev):
         right = K.gemm(x, w[:, 2048:].contiguous(), None if b_ is None else b_[2048:].contiguous(), relu)
         assert torch.equal(y[..., :2048], left) and torch.equal(y[..., 2048:], right)
         assert_close(y, R.linear(x, w, b_, relu), name="y")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("case", [
+    # (la, lb, M, N, K, what the library does with it)
+    (0, 1, 100, 333, 129, "ragged, K not a multiple of 64: register-staged kernel"),
+    (0, 0, 77, 136, 264, "unaligned leading dimensions cannot occur here, odd extents do: register-staged kernel"),
+    (1, 1, 256, 256, 8192, "one tile, long contraction: split over workgroups, scaled in the reduce pass"),
+    (0, 1, 8192, 3072, 1024, "1.5 rounds of tiles: cut along N into whole rounds + tail"),
+    (0, 0, 512, 1024, 4096, "direct-to-LDS kernel, scaled in its write-out"),
+])
+def test_gemm_scaled_is_alpha_times_the_product(case, dtype, dev):
+    """tf_gemm_scaled multiplies the fp32 sums by a device-resident scalar in whichever write-out the
+    product takes (register-staged kernel, direct-to-LDS kernel, reduce pass of a split contraction,
+    both halves of a product cut along N): against tf_gemm_out with an fp32 result scaled afterwards,
+    for fp32 and for 16-bit output.  The factor is applied before the single rounding, so both
+    comparisons are exact."""
+    la, lb, M, N, K, _ = case
+    g = torch.Generator().manual_seed(41)
+    a = torch.randn((M, K) if la == 0 else (K, M), generator=g).to(dtype).to(dev)
+    b = (torch.randn((N, K) if lb == 0 else (K, N), generator=g) / K ** 0.5).to(dtype).to(dev)
+    alpha = torch.tensor([0.3173], dtype=torch.float32, device=dev)
+    plain = torch.empty((M, N), dtype=torch.float32, device=dev)
+    K_mod._gemm(dtype, la, lb, M, N, K, a, a.stride(0), b, b.stride(0), plain, N, None, False)
+    want = (a.float() if la == 0 else a.float().T) @ (b.float().T if lb == 0 else b.float())
+    assert rel_l2(plain, want) < 1e-3
+    for out_dtype in (torch.float32, dtype):
+        out = torch.full((M, N), float("nan"), dtype=out_dtype, device=dev)
+        K_mod.gemm_scaled(a, la, M, K, a.stride(0), b, lb, N, b.stride(0), alpha, out)
+        assert torch.equal(out, (plain * alpha).to(out_dtype)), (case, out_dtype)

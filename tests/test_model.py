@@ -201,10 +201,11 @@ def _layer_case(name, dev, share_relu_mask=False):
     return dtype == torch.float16, loss.item(), loss_ref.item(), errs
 
 
-@pytest.mark.parametrize("name", [n for n in FULL_SIZE if "410M" not in n])
+@pytest.mark.parametrize("name", list(FULL_SIZE))
 def test_full_size_layer_against_cpu_oracle(name, dev):
     """One TransformerLayer + final LayerNorm + LM head + shifted cross-entropy at the real
-    d / ffn / heads / head_dim / bias / ALiBi / ctx / batch of baseline configurations 2, 4 and 5
+    d / ffn / heads / head_dim / bias / ALiBi / ctx / batch of baseline configurations 2, 3 (the headline
+    410M shape: packed q/k/v product 8192 x 3072, grouped weight gradients, fused LM head at d = 1024), 4 and 5
     (fp16 and bf16), every gradient compared with the fp32 oracle running on the CPU.  The LM head
     and the cross-entropy see the last 512 / B + 1 positions of every sequence (512 loss rows in
     all); a second loss term, a fixed random linear functional of the final LayerNorm's output at

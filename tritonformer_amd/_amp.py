@@ -55,7 +55,9 @@ def cached_conversion(weights, dtype, convert):
     if hit is not None and hit[1] == state and all(r() is w for r, w in zip(hit[0], weights)):
         return hit[2]
     out = convert(weights, dtype)
-    _cache[key] = (tuple(weakref.ref(w) for w in weights), state, out)
+    # the entry (and the 16-bit copy it holds) goes when any of its parameters does
+    refs = tuple(weakref.ref(w, lambda _, key=key: _cache.pop(key, None)) for w in weights)
+    _cache[key] = (refs, state, out)
     return out
 
 

@@ -1250,7 +1250,9 @@ static int gemm_entry(void* stream, int dtype, int out_dtype, int layout_a, int 
   }
   const GemmPlan pl = make_plan(M, N, K, vec, mask_act == nullptr && !signs, nullptr, force);
   // the sign bits exist in the write-out of the direct-to-LDS kernels only
-  if (signs && !(kCfgs[pl.cfg].dma && vec && K % pl.bk == 0 && pl.splits == 1)) return TF_EINVAL;
+  // (TF_ESHAPE, so that a caller can tell "this product is not served, use the activation as mask"
+  // from a malformed call)
+  if (signs && !(kCfgs[pl.cfg].dma && vec && K % pl.bk == 0 && pl.splits == 1)) return TF_ESHAPE;
   const int64_t need = pl.splits > 1 ? (int64_t)pl.splits * M * N * (int64_t)sizeof(float) : 0;
   if (need > 0 && (!workspace || workspace_bytes < need)) return TF_EWORKSPACE;
   if (need > 0 && !aligned16(workspace)) return TF_EALIGN;

@@ -97,6 +97,9 @@ def gemm(a, b, bias=None, fuse_relu=False, mask_act=None):
     return out
 
 
+_BITS_NOT_SERVED = -4  # TF_ESHAPE from tf_gemm_relu_bits: the product misses the bit kernel's preconditions
+
+
 def _gemm_bits(dtype, lb, m, n, k, a, b, ldb, c, bias, bits_out, bits_in):
     """One tf_gemm_relu_bits call (A contraction-contiguous); returns the status code."""
     return load().tf_gemm_relu_bits(stream_ptr(), dtype_code(dtype), dtype_code(dtype), KMAJOR, lb, m, n, k,
@@ -123,6 +126,8 @@ def gemm_relu_bits(a, b, bias=None):
         rc = _gemm_bits(a.dtype, lb, m, n, k, a2, b, ldb, out, bias, bits, None)
         if rc == 0:
             return out, bits
+        if rc != _BITS_NOT_SERVED:
+            check(rc)
     _gemm(a.dtype, KMAJOR, lb, m, n, k, a2, k, b, ldb, out, n, bias, True, None)
     return out, None
 
@@ -141,8 +146,8 @@ def mm_masked_bits(a, b, bits, act=None):
     b, lb, ldb = _operand_b(b, n, k)
     out = torch.empty(a.shape[:-1] + (n,), dtype=a.dtype, device=a.device)
     rc = _gemm_bits(a.dtype, lb, m, n, k, a2, b, ldb, out, None, None, bits)
-    if rc != 0 and act is not None:
-        return gemm(a, b, None, False, act)
+    if rc == _BITS_NOT_SERVED and act is not None:
+        return gemm(a, b, None, False, act)  # any other status is an error and is raised below
     check(rc)
     return out
 
@@ -404,6 +409,8 @@ def flash_wrapper_fwd(q, k, v, bias=None, out=None):
     kernels/biased_attention.py:188-245); (B, nh, S + 32) when S is not a multiple of 64."""
     _check_attn(q, k, v, bias)
     b, nh, s, hd = q.shape
+    if out is not None and (out.shape != q.shape or out.dtype != q.dtype or not _strided_ok(out)):
+        raise ValueError("attention output buffer must match q in shape and dtype, with aligned strides")
     if s % 64:
         # head_dim 128 with S = 32 (mod 64), which the reference serves with 32-row blocks: the
         # kernels work on 64-row blocks, so the sequence is continued by 32 rows of zeros.  Under
@@ -418,8 +425,6 @@ def flash_wrapper_fwd(q, k, v, bias=None, out=None):
     q, k, v = _attn_layout(q, k, v)
     if out is None:
         out = torch.empty_strided(q.shape, q.stride(), dtype=q.dtype, device=q.device)
-    elif out.shape != q.shape or out.dtype != q.dtype or not _strided_ok(out):
-        raise ValueError("attention output buffer must match q in shape and dtype, with aligned strides")
     lse = torch.empty((b, nh, s), dtype=torch.float32, device=q.device)
     if bias is not None and bias.ndim == 1:
         slopes = bias.contiguous()
