@@ -553,6 +553,95 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x16 (&
   }
 }
 
+// One bit per element of a chunk of eight 16-bit values none of which is negative (a ReLU output;
+// -0 counts as zero): bit e set where element e is positive.  Word arithmetic on the packed
+// halves: h & 0x7fff is 0 or at least 1, so (h & 0x7fff) + 0x7fff carries into bit 15 exactly
+// for the positive ones (and never into the neighbouring half).
+__device__ __forceinline__ unsigned positive_bits8(u32x4 v) {
+  unsigned b = 0;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const unsigned t = ((v[k] & 0x7fff7fffu) + 0x7fff7fffu) >> 15 & 0x00010001u;  // elements 2k (bit 0), 2k+1 (bit 16)
+    b |= t << (2 * k);
+  }
+  return (b | b >> 15) & 0xffu;
+}
+// ... and the reverse: the chunk with every element whose bit is clear set to zero
+__device__ __forceinline__ u32x4 keep_by_bits8(u32x4 v, unsigned bits) {
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const unsigned lo = (unsigned)__builtin_amdgcn_sbfe((int)bits, 2 * k, 1);      // 0 or 0xffffffff
+    const unsigned hi = (unsigned)__builtin_amdgcn_sbfe((int)bits, 2 * k + 1, 1);
+    v[k] &= __builtin_amdgcn_perm(hi, lo, 0x05040100u);  // bytes: lo.0 lo.1 hi.0 hi.1
+  }
+  return v;
+}
+
+// Write-out of a full tile with the ReLU sign bits, 16-bit result, no tests in the store loop.
+//  BITS_OUT: C = relu(acc + bias), bits = (C > 0).  A lane's bit bytes go to an LDS image of the
+//            tile's bits (BM rows of BN / 8 bytes) and leave it as whole 16-byte pieces after a
+//            barrier: stored from the loop they would be 64 single bytes per store instruction,
+//            eight to a row, a partial write of eight lines each.
+//  !BITS_OUT: C = bit ? acc : 0, the bytes requested before the main loop (sign_bytes).
+template <typename T, int BM, int BN, int TM, int TN, int WTM, int WTN, bool BITS_OUT>
+__device__ __forceinline__ void gemm_epilogue_bits(const GemmParams& p, f32x16 (&acc)[TM][TN], char* smem, int m0, int n0,
+                                                   int wm, int wn, int wave, int lane, const uint8_t (*sign_bytes)[4]) {
+  constexpr int ROWB = WTN * 2 + 16, CH = WTN * 2 / 16, RPI = 64 / CH;
+  constexpr int NW = (BM / WTM) * (BN / WTN);
+  constexpr int IMG = NW * 32 * ROWB;  // the bit image lies behind the waves' slabs
+  static_assert(BN / 8 % 16 == 0, "rows of the bit image are whole 16-byte pieces");
+  char* mine = smem + wave * (32 * ROWB);
+  const T* bias = (const T*)p.bias;
+  T* C = (T*)p.C;
+  const int nbase = n0 + wn * WTN;
+  const int n_lane = nbase + (lane % CH) * 8;
+  T* const row0 = C + (int64_t)(m0 + wm * WTM + lane / CH) * p.ldc + n_lane + (int64_t)(n_lane / p.chunk_n) * p.chunk_skip;
+  typename Vec<T>::v4 bvals[TN][4] = {};
+  if (BITS_OUT && bias) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) bvals[j][g] = *reinterpret_cast<const typename Vec<T>::v4*>(bias + nbase + j * 32 + g * 8 + (lane >> 5) * 4);
+  }
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        typename Vec<T>::v4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float v = acc[i][j][g * 4 + e];
+          if (BITS_OUT) v = fmaxf(v + (float)bvals[j][g][e], 0.f);
+          o[e] = (T)v;
+        }
+        *reinterpret_cast<typename Vec<T>::v4*>(mine + (lane & 31) * ROWB + (j * 32 + g * 8 + (lane >> 5) * 4) * 2) = o;
+      }
+    u32x4 vals[32 / RPI];
+#pragma unroll
+    for (int rr = 0; rr < 32 / RPI; ++rr) vals[rr] = lds_ld16(mine, (rr * RPI + lane / CH) * ROWB + (lane % CH) * 16);
+#pragma unroll
+    for (int rr = 0; rr < 32 / RPI; ++rr) {
+      u32x4 val = vals[rr];
+      if (BITS_OUT) {
+        const int row = wm * WTM + i * 32 + rr * RPI + lane / CH;  // in the tile
+        smem[IMG + row * (BN / 8) + wn * (WTN / 8) + lane % CH] = (char)positive_bits8(val);
+      } else {
+        val = keep_by_bits8(val, sign_bytes[i][rr]);
+      }
+      st16(row0 + (int64_t)(i * 32 + rr * RPI) * p.ldc, val);
+    }
+  }
+  if (BITS_OUT) {
+    __syncthreads();
+    constexpr int PIECES = BM * (BN / 8) / 16, PPR = BN / 8 / 16;  // 16-byte pieces of the image, per row
+    uint8_t* out = (uint8_t*)p.sign_out + (int64_t)m0 * p.ldsign + n0 / 8;
+    for (int q = threadIdx.x; q < PIECES; q += NW * 64)
+      *reinterpret_cast<u32x4*>(out + (int64_t)(q / PPR) * p.ldsign + (q % PPR) * 16) = lds_ld16(smem, IMG + q * 16);
+  }
+}
+
 template <typename T, int BM, int BN, int BK, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR>
 __device__ __forceinline__ void gemm_dma_body(const GemmParams& p, const int pid) {
   constexpr int NW = WM * WN;
@@ -737,6 +826,7 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams& p, const int pid
   if (kt < nk) stage(smem + (kt & 1) * STAGE, smem + ((kt + 1) & 1) * STAGE, no_t(), no_t());
 
   static_assert(NW * 32 * (WTN * 4 + 16) <= 2 * STAGE, "epilogue staging must fit in the pipeline LDS");
+  static_assert(NW * 32 * (WTN * 2 + 16) + BM * BN / 8 <= 2 * STAGE, "... and so must the image of a tile's sign bits behind it");
   const bool full = m0 + BM <= p.M && n0 + BN <= p.N;  // no row or column of the tile lies outside C: stores need no test
   if (p.splits > 1) {
     // fp32 partial of this contraction slice: a plain (M, N) matrix, written like an fp32 result
@@ -762,8 +852,18 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams& p, const int pid
       else if (plain) gemm_epilogue_lds<T, float, TM, TN, WTM, WTN, true>(p, acc, smem, m0, n0, wm, wn, wave, lane);
       else gemm_epilogue_lds<T, float, TM, TN, WTM, WTN>(p, acc, smem, m0, n0, wm, wn, wave, lane);
     } else {
+      // the two sign-bit launches of a fused MLP, on full tiles of a plain (unchunked) result whose bit rows take
+      // 16-byte pieces: write-outs of their own, nothing tested per store
+#ifdef TF_NO_FAST_BITS
+      const bool bits_fast = false &&
+#else
+      const bool bits_fast = full &&
+#endif !p.mask && !p.alpha && p.chunk_skip == 0 && p.ldsign % 16 == 0 &&
+                             (reinterpret_cast<uintptr_t>(p.sign_out) & 15) == 0;
       if (plain && full) gemm_epilogue_lds<T, T, TM, TN, WTM, WTN, true, true>(p, acc, smem, m0, n0, wm, wn, wave, lane);
       else if (plain) gemm_epilogue_lds<T, T, TM, TN, WTM, WTN, true>(p, acc, smem, m0, n0, wm, wn, wave, lane);
+      else if (bits_fast && p.sign_out && p.relu) gemm_epilogue_bits<T, BM, BN, TM, TN, WTM, WTN, true>(p, acc, smem, m0, n0, wm, wn, wave, lane, sign_bytes);
+      else if (bits_fast && p.sign_in && !p.bias && !p.relu) gemm_epilogue_bits<T, BM, BN, TM, TN, WTM, WTN, false>(p, acc, smem, m0, n0, wm, wn, wave, lane, sign_bytes);
       else gemm_epilogue_lds<T, T, TM, TN, WTM, WTN>(p, acc, smem, m0, n0, wm, wn, wave, lane, sign_bytes);
     }
   }
