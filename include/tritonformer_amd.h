@@ -174,11 +174,11 @@ int64_t tf_gemm_group_workspace_bytes(int layout_a, int layout_b, int count,
  * (kernels/biased_attention.py:101-106); -inf entries are allowed.
  * Replaces flash_wrapper_fwd (kernels/attention.py:171-217) and
  * flash_wrapper_fwd_attn_bias (kernels/biased_attention.py:188-245).
- * Preconditions: hd in {32,64,128} (as the reference asserts); S % 64 == 0.  The reference
- * asserts S % 64 == 0 too, except at hd = 128, where its 32-row blocks admit S % 32 == 0
- * (kernels/attention.py:177-183); a caller with such a length continues q, k, v with 32 rows
- * of zeros (under the causal mask no real query sees them) and drops the added output rows,
- * as the Python launcher of this package does. */
+ * Preconditions: hd in {32,64,128} (as the reference asserts); S % 32 == 0.  The reference
+ * asserts S % 64 == 0, except at hd = 128, where its 32-row blocks admit S % 32 == 0
+ * (kernels/attention.py:177-183); here every head_dim takes S % 32 == 0 (64-row blocks, the
+ * last one of a sequence half used).  Nothing beyond row S - 1 of q, k, v, o, lse or of the
+ * bias rows is read or written. */
 int tf_attn_fwd(void* stream, int dtype, int64_t B, int64_t nh, int64_t S, int64_t hd,
                 const void* q, const void* k, const void* v, void* o,
                 int64_t sb, int64_t sh, int64_t ss, int64_t osb, int64_t osh, int64_t oss,

@@ -208,7 +208,7 @@ def test_attention_rejects_bad_shapes():
         return lib.tf_attn_fwd(None, dtype, 1, 2, S, hd, FAKE, FAKE, FAKE, FAKE, S * 2 * hd, hd, row, S * 2 * hd, hd,
                                2 * hd, FAKE, bias, bsr * bsr if bias else 0, bsr, 0.125)
 
-    assert fwd(100, 64) == -4           # S % 64 != 0
+    assert fwd(100, 64) == -4           # S % 32 != 0
     assert fwd(128, 48) == -4           # head_dim not in {32, 64, 128}
     assert fwd(128, 64, dtype=2) == -2  # fp32
     assert fwd(128, 64, ss=60) == -3    # row stride not a multiple of 8 elements

@@ -203,3 +203,73 @@ def test_attention_block_equals_separate_functions(use_bias, dev):
     assert torch.equal(y1, y0) and torch.equal(dx1, dx0)
     for a, c in zip(dw1, dw0):
         assert a.shape == (d, d) and a.is_contiguous() and rel_l2(a, c) < 1e-3
+
+
+@pytest.mark.parametrize("dims", [(2, 3, 96, 64), (1, 2, 160, 32), (1, 4, 32, 64), (2, 2, 224, 128), (1, 2, 1056, 64)])
+@pytest.mark.parametrize("bias_kind", ["none", "dense", "alibi"])
+def test_half_used_last_block_through_the_c_abi(dims, bias_kind, dev):
+    """S = 32 (mod 64) at every head_dim: the kernels walk 64-row blocks and use half of the last one.  The
+    operator keeps the reference's rule (multiples of 64 below head_dim 128), so these go through the C
+    ABI directly.  q, k, v, o, dO, lse and the dense bias lie in buffers whose every element beyond the
+    sequence is NaN: a row of the unused half that took part in anything would show in the results."""
+    import math
+    from tritonformer_amd import _lib
+    from tritonformer_amd.transformer import get_slopes
+
+    lib = _lib.load()
+    b, nh, s, hd = dims
+    g = torch.Generator().manual_seed(5)
+    nan = float("nan")
+
+    def poisoned(*shape):
+        """(B, S, nh, hd)-shaped random data at the front of a NaN buffer with 64 spare rows behind every sequence"""
+        buf = torch.full((b, s + 64, nh, hd), nan, dtype=torch.float16)
+        buf[:, :s] = torch.randn(b, s, nh, hd, generator=g).half()
+        return buf.to(dev)
+
+    qb, kb, vb, dob = poisoned(), poisoned(), poisoned(), poisoned()
+    ob, dqb, dkb, dvb = (torch.full((b, s + 64, nh, hd), nan, dtype=torch.float16, device=dev) for _ in range(4))
+    lse = torch.full((b * nh * s + 64,), nan, dtype=torch.float32, device=dev)
+    delta = torch.full((b * nh * s + 64,), nan, dtype=torch.float32, device=dev)
+    sb, sh, ss = (s + 64) * nh * hd, hd, nh * hd
+    bias_t = slopes = None
+    bias_ref = None
+    if bias_kind == "dense":
+        sp = s  # exactly the sequence: nothing to spare behind the last row or column
+        bias_full = torch.full((nh, sp + 8, sp + 8), nan, dtype=torch.float16)
+        bias_ref = (torch.randn(nh, sp, sp, generator=g) * 0.5).half()
+        bias_full[:, :sp, :sp] = bias_ref
+        bias_t = bias_full.to(dev)
+    elif bias_kind == "alibi":
+        slopes = torch.tensor(get_slopes(nh), dtype=torch.float16, device=dev)
+        bias_ref = R.alibi_mask(s, nh)
+    stream = torch.cuda.current_stream().cuda_stream
+    scale = 1.0 / math.sqrt(hd)
+    if slopes is not None:
+        _lib.check(lib.tf_attn_alibi_fwd(stream, 0, b, nh, s, hd, qb.data_ptr(), kb.data_ptr(), vb.data_ptr(), ob.data_ptr(),
+                                         sb, sh, ss, sb, sh, ss, lse.data_ptr(), slopes.data_ptr(), scale))
+        _lib.check(lib.tf_attn_alibi_bwd(stream, 0, b, nh, s, hd, qb.data_ptr(), kb.data_ptr(), vb.data_ptr(), ob.data_ptr(),
+                                         dob.data_ptr(), dqb.data_ptr(), dkb.data_ptr(), dvb.data_ptr(), sb, sh, ss, sb, sh, ss,
+                                         lse.data_ptr(), delta.data_ptr(), slopes.data_ptr(), scale))
+    else:
+        bargs = (bias_t.data_ptr(), bias_t.stride(0), bias_t.stride(1)) if bias_t is not None else (None, 0, 0)
+        _lib.check(lib.tf_attn_fwd(stream, 0, b, nh, s, hd, qb.data_ptr(), kb.data_ptr(), vb.data_ptr(), ob.data_ptr(),
+                                   sb, sh, ss, sb, sh, ss, lse.data_ptr(), *bargs, scale))
+        _lib.check(lib.tf_attn_bwd(stream, 0, b, nh, s, hd, qb.data_ptr(), kb.data_ptr(), vb.data_ptr(), ob.data_ptr(),
+                                   dob.data_ptr(), dqb.data_ptr(), dkb.data_ptr(), dvb.data_ptr(), sb, sh, ss, sb, sh, ss,
+                                   lse.data_ptr(), delta.data_ptr(), *bargs, scale))
+    torch.cuda.synchronize()
+    view = lambda t: t[:, :s].permute(0, 2, 1, 3)
+    qr, kr, vr = (view(t).float().cpu().requires_grad_(True) for t in (qb, kb, vb))
+    o_ref = R.causal_attention(qr, kr, vr, bias_ref)
+    o_ref.backward(view(dob).float().cpu())
+    tag = f"{dims} {bias_kind}"
+    assert_close(view(ob), o_ref, name="o " + tag)
+    assert_close(view(dqb), qr.grad, name="dq " + tag)
+    assert_close(view(dkb), kr.grad, name="dk " + tag)
+    assert_close(view(dvb), vr.grad, name="dv " + tag)
+    # nothing was written behind the sequences
+    for t in (ob, dqb, dkb, dvb):
+        assert torch.isnan(t[:, s:]).all()
+    assert torch.isnan(lse[b * nh * s:]).all() and torch.isnan(delta[b * nh * s:]).all()
+    assert torch.isfinite(lse[: b * nh * s]).all()

@@ -70,6 +70,16 @@ struct SeqTile {
       ptr[j] = base + (int64_t)(row0 + row) * ss + c * 8;
     }
   }
+  // A sequence may end half way through a 64-row block (S = 32 mod 64).  Before the loads of that last
+  // block, the pointers of its rows 32 .. 63 -- which lie beyond the sequence, possibly beyond the
+  // allocation -- are moved 32 rows back: the tile then holds rows 0 .. 31 twice.  No valid query ever
+  // sees the copies (keys beyond the sequence lie above every diagonal; queries beyond it are skipped),
+  // they only have to be readable and finite.
+  static __device__ __forceinline__ void stream_tail(const T* (&ptr)[PER_THREAD], int64_t ss) {
+#pragma unroll
+    for (int j = 0; j < PER_THREAD; ++j)
+      if ((int)threadIdx.x + j * 256 >= 32 * CPR) ptr[j] -= 32 * ss;
+  }
   // LDS destination of a wave's j-th load into the tile at `tile`
   static __device__ __forceinline__ char* stream_slot(char* tile, int wave, int j) {
     return tile + (j * 256 + wave * 64) * 16;
@@ -155,6 +165,15 @@ struct BiasTile {
       bp[j] = bias_head + (int64_t)qrow * row_stride + c * 8;
     }
   }
+  // last block of a sequence that ends half way through it: chunks of key columns 32 .. 63 read 32 columns back
+  template <typename T> static __device__ __forceinline__ void tail(const T* (&bp)[4]) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int id = threadIdx.x + j * 256;
+      const int row = id >> 3, c = (id & 7) ^ ((row >> 1) & 7);
+      if (c >= 4) bp[j] -= 32;
+    }
+  }
   // next 64 keys into the tile at `dst`; advances the pointers
   template <typename T> static __device__ __forceinline__ void load(const T* (&bp)[4], char* dst, int wave) {
 #pragma unroll
@@ -220,7 +239,7 @@ __device__ __forceinline__ void store_rows32(char* slab, T* dst, int64_t row_str
 // ===========================================================================
 constexpr float kRescaleThreshold = 8.0f;  // log2 domain
 
-template <typename T, int HD, int BMODE>
+template <typename T, int HD, int BMODE, bool TAIL>
 __global__ __launch_bounds__(256, HD > 64 ? 1 : (BMODE == kDenseBias ? 2 : 3)) void attn_fwd_kernel(AttnParams p) {
   constexpr bool HAS_BIAS = BMODE == kDenseBias, ALIBI = BMODE == kAlibi;
   typedef SeqTile<T, 64, HD> KT;
@@ -251,7 +270,7 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (BMODE == kDenseBias ? 2 : 3)) v
   const bool active = q0w < p.S;
   const int myq = q0w + (lane & 31);
   const int kv_end = min(p.S, q0 + 128);
-  const int nkv = kv_end / 64;
+  const int nkv = (kv_end + 63) / 64;  // the last block may be half beyond the sequence (S = 32 mod 64)
 
   v8 qf[KS];
 #pragma unroll
@@ -289,18 +308,27 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (BMODE == kDenseBias ? 2 : 3)) v
     }
     if (HAS_BIAS) BiasTile::load(bp, smem + stage_off + 2 * KT::BYTES, wave_u);
   };
+  // the loads of key block jb: if the sequence ends inside it (TAIL: S = 32 mod 64, an instantiation of its
+  // own, so that whole-block sequences pay nothing), rows / bias columns 32 .. 63 are taken 32 earlier
+  auto load_block_of = [&](int jb, int stage_off) {
+    if (TAIL && (jb + 1) * 64 > p.S) {
+      KT::stream_tail(kp, p.ss);
+      if (HAS_BIAS) BiasTile::tail(bp);
+    }
+    load_tile(stage_off);
+  };
   uint32_t ka[KS], va[DT][2];
   const uint32_t lds0 = lds_address(smem);
   KT::operand_addrs(ka, va, lds0, lane);
 
-  load_tile(0);
+  load_block_of(0, 0);
   __syncthreads();
 
   // One 64-key block out of the stage at byte offset SOFF.
   auto step = [&](auto stage_tag, int j) {
     constexpr int SOFF = decltype(stage_tag)::value * STAGE;
     constexpr int VOFF = SOFF + KT::BYTES;
-    if (j + 1 < nkv) load_tile(STAGE - SOFF);
+    if (j + 1 < nkv) load_block_of(j + 1, STAGE - SOFF);
     const int kb = j * 64;
     if (active && kb <= q0w + 31) {
       auto block = [&](auto diag_tag) {
@@ -428,7 +456,7 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (BMODE == kDenseBias ? 2 : 3)) v
 // dK/dV pass.  Workgroup: 4 waves x 32 keys; query blocks of 64 from the
 // diagonal downwards.  Q and dO tiles (+ their lse / delta) go through LDS.
 // ===========================================================================
-template <typename T, int HD, int BMODE>
+template <typename T, int HD, int BMODE, bool TAIL>
 __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_dkdv_kernel(AttnParams p) {
   constexpr bool HAS_BIAS = BMODE == kDenseBias, ALIBI = BMODE == kAlibi;
   typedef SeqTile<T, 64, HD> QT;
@@ -478,7 +506,7 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_dkdv_kernel(AttnPa
 #pragma unroll
     for (int r = 0; r < 16; ++r) { dk[d][r] = 0.f; dv[d][r] = 0.f; }
 
-  const int nq = (p.S - k0) / 64;  // query blocks k0, k0+64, ...
+  const int nq = (p.S - k0 + 63) / 64;  // query blocks k0, k0+64, ...; the last one may be half beyond the sequence
 
   // Everything a query block needs goes from global memory straight into LDS: the Q and dO
   // tiles (chunk swizzle on the global side), the two statistics rows (one float per lane of
@@ -528,18 +556,34 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_dkdv_kernel(AttnPa
   const uint32_t sa = lds0 + STAT + 16 * (lane >> 5);  // statistics of queries g*8 + 4*(lane/32) .. +3
   const uint32_t ba = lds0 + BIAS + (4 * (lane >> 5)) * 256 + (wave * 32 + (lane & 31)) * 2;
 
-  if (nq > 0) load_block(0);
+  // the loads of query block ib: if the sequence ends inside it, its rows 32 .. 63 (tiles, statistics, bias rows)
+  // are taken 32 earlier; the sub-tile they fill is never used
+  auto load_block_of = [&](int ib, int stage_off) {
+    if (TAIL && k0 + (ib + 1) * 64 > p.S) {
+      QT::stream_tail(qp, p.ss);
+      QT::stream_tail(dop, p.oss);
+      if (lane >= 32) statp -= 32;
+      if (HAS_BIAS) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (((threadIdx.x + j * 256) >> 4) >= 32) bp[j] -= (int64_t)32 * p.bias_sr;
+      }
+    }
+    load_block(stage_off);
+  };
+  if (nq > 0) load_block_of(0, 0);
   __syncthreads();
 
   auto step = [&](auto stage_tag, int it) {
     constexpr int SOFF = decltype(stage_tag)::value * STAGE;
-    if (it + 1 < nq) load_block(STAGE - SOFF);
+    if (it + 1 < nq) load_block_of(it + 1, STAGE - SOFF);
     const int qb = k0 + it * 64;
     if (active) {
       static_for<2>([&](auto qt_tag) {
         constexpr int qt = decltype(qt_tag)::value;
         const int qs = qb + qt * 32;      // first query of this 32-row sub-tile
         if (qs + 31 < kw0) return;        // entirely above the diagonal for this wave
+        if (TAIL && qs >= p.S) return;    // beyond the sequence (the second half of its last block)
         auto tile = [&](auto diag_tag) {
           constexpr bool DIAG = decltype(diag_tag)::value;
           constexpr int ROFF = SOFF + qt * 32 * HD * 2;
@@ -656,7 +700,7 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_dkdv_kernel(AttnPa
 // dQ pass.  Workgroup: 4 waves x 32 queries; key/value blocks of 64 up to the
 // diagonal, K and V tiles through LDS.
 // ===========================================================================
-template <typename T, int HD, int BMODE>
+template <typename T, int HD, int BMODE, bool TAIL>
 __global__ __launch_bounds__(256, HD > 64 ? 1 : (BMODE != kNoBias ? 2 : 3)) void attn_dq_kernel(AttnParams p) {
   constexpr bool HAS_BIAS = BMODE == kDenseBias, ALIBI = BMODE == kAlibi;
   typedef SeqTile<T, 64, HD> KT;
@@ -686,7 +730,7 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (BMODE != kNoBias ? 2 : 3)) void
   const bool active = q0w < p.S;
   const int myq = q0w + (lane & 31);
   const int kv_end = min(p.S, q0 + 128);
-  const int nkv = kv_end / 64;
+  const int nkv = (kv_end + 63) / 64;  // the last block may be half beyond the sequence (S = 32 mod 64)
 
   v8 qf[KS], dof[KS];
   float neg_lse = 0.f, neg_delta = 0.f;
@@ -741,17 +785,26 @@ __global__ __launch_bounds__(256, HD > 64 ? 1 : (BMODE != kNoBias ? 2 : 3)) void
     }
     if (HAS_BIAS) BiasTile::load(bp, smem + stage_off + 2 * KT::BYTES, wave_u);
   };
+  // the loads of key block jb: if the sequence ends inside it (TAIL: S = 32 mod 64, an instantiation of its
+  // own, so that whole-block sequences pay nothing), rows / bias columns 32 .. 63 are taken 32 earlier
+  auto load_block_of = [&](int jb, int stage_off) {
+    if (TAIL && (jb + 1) * 64 > p.S) {
+      KT::stream_tail(kp, p.ss);
+      if (HAS_BIAS) BiasTile::tail(bp);
+    }
+    load_tile(stage_off);
+  };
   // row operands of K and V, hd operands of K
   uint32_t ra[KS], ha[DT][2];
   const uint32_t lds0 = lds_address(smem);
   KT::operand_addrs(ra, ha, lds0, lane);
 
-  load_tile(0);
+  load_block_of(0, 0);
   __syncthreads();
 
   auto step = [&](auto stage_tag, int j) {
     constexpr int SOFF = decltype(stage_tag)::value * STAGE;
-    if (j + 1 < nkv) load_tile(STAGE - SOFF);
+    if (j + 1 < nkv) load_block_of(j + 1, STAGE - SOFF);
     const int kb = j * 64;
     if (active) {
       static_for<2>([&](auto jt_tag) {
@@ -858,10 +911,10 @@ static void allow_lds(K kernel, int bytes) {
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
 }
 
-template <typename T, int HD, int MODE>
+template <typename T, int HD, int MODE, bool TAIL>
 static int fwd_launch(hipStream_t st, const AttnParams& p) {
   constexpr int lds = 2 * (2 * SeqTile<T, 64, HD>::BYTES + (MODE == kDenseBias ? BiasTile::BYTES : 0));
-  auto kernel = attn_fwd_kernel<T, HD, MODE>;
+  auto kernel = attn_fwd_kernel<T, HD, MODE, TAIL>;
   static bool once = (allow_lds(kernel, lds), true);
   (void)once;
   const unsigned grid = (unsigned)(((p.S + 127) / 128) * p.B * p.nh);
@@ -871,12 +924,12 @@ static int fwd_launch(hipStream_t st, const AttnParams& p) {
 }
 
 // dQ pass first: it also produces the -delta rows that the dK/dV pass reads.
-template <typename T, int HD, int MODE>
+template <typename T, int HD, int MODE, bool TAIL>
 static int bwd_launch(hipStream_t st, const AttnParams& p) {
   const unsigned grid = (unsigned)(((p.S + 127) / 128) * p.B * p.nh);
   {
     constexpr int lds = 2 * (2 * SeqTile<T, 64, HD>::BYTES + (MODE == kDenseBias ? BiasTile::BYTES : 0));
-    auto kernel = attn_dq_kernel<T, HD, MODE>;
+    auto kernel = attn_dq_kernel<T, HD, MODE, TAIL>;
     static bool once = (allow_lds(kernel, lds), true);
     (void)once;
     kernel<<<dim3(grid), dim3(256), lds, st>>>(p);
@@ -884,7 +937,7 @@ static int bwd_launch(hipStream_t st, const AttnParams& p) {
   }
   {
     constexpr int lds = 2 * (2 * SeqTile<T, 64, HD>::BYTES + 2 * 64 * 4 + (MODE == kDenseBias ? 64 * 128 * 2 : 0));
-    auto kernel = attn_dkdv_kernel<T, HD, MODE>;
+    auto kernel = attn_dkdv_kernel<T, HD, MODE, TAIL>;
     static bool once = (allow_lds(kernel, lds), true);
     (void)once;
     kernel<<<dim3(grid), dim3(256), lds, st>>>(p);
@@ -893,14 +946,20 @@ static int bwd_launch(hipStream_t st, const AttnParams& p) {
   return TF_OK;
 }
 
-template <typename T, bool FWD, int MODE>
-static int attn_dispatch_hd(hipStream_t st, int hd, const AttnParams& p) {
+template <typename T, bool FWD, int MODE, bool TAIL>
+static int attn_dispatch_tail(hipStream_t st, int hd, const AttnParams& p) {
   switch (hd) {
-    case 32: return FWD ? fwd_launch<T, 32, MODE>(st, p) : bwd_launch<T, 32, MODE>(st, p);
-    case 64: return FWD ? fwd_launch<T, 64, MODE>(st, p) : bwd_launch<T, 64, MODE>(st, p);
-    case 128: return FWD ? fwd_launch<T, 128, MODE>(st, p) : bwd_launch<T, 128, MODE>(st, p);
+    case 32: return FWD ? fwd_launch<T, 32, MODE, TAIL>(st, p) : bwd_launch<T, 32, MODE, TAIL>(st, p);
+    case 64: return FWD ? fwd_launch<T, 64, MODE, TAIL>(st, p) : bwd_launch<T, 64, MODE, TAIL>(st, p);
+    case 128: return FWD ? fwd_launch<T, 128, MODE, TAIL>(st, p) : bwd_launch<T, 128, MODE, TAIL>(st, p);
   }
   return TF_ESHAPE;
+}
+template <typename T, bool FWD, int MODE>
+static int attn_dispatch_hd(hipStream_t st, int hd, const AttnParams& p) {
+  // a sequence that ends half way through its last 64-row block takes kernels of its own
+  if (p.S % 64) return attn_dispatch_tail<T, FWD, MODE, true>(st, hd, p);
+  return attn_dispatch_tail<T, FWD, MODE, false>(st, hd, p);
 }
 
 template <typename T, bool FWD>
@@ -915,10 +974,10 @@ static int attn_check(int dtype, int64_t B, int64_t nh, int64_t S, int64_t hd, i
   if (dtype != TF_F16 && dtype != TF_BF16) return TF_EDTYPE;
   if (B <= 0 || nh <= 0 || S <= 0) return TF_EINVAL;
   if (hd != 32 && hd != 64 && hd != 128) return TF_ESHAPE;  // as kernels/attention.py:567
-  // 64-row blocks for every head_dim (the reference, kernels/attention.py:177-183, uses 32-row
-  // blocks at head_dim 128 and so accepts S % 32 == 0 there: the Python launcher serves those
-  // lengths by continuing the sequence with 32 rows of zeros)
-  if (S % 64 != 0) return TF_ESHAPE;
+  // 64-row blocks for every head_dim, the last one of a sequence half used when S = 32 (mod 64): the
+  // reference (kernels/attention.py:177-183) uses 32-row blocks at head_dim 128 and so takes
+  // S % 32 == 0 there; here every head_dim does
+  if (S % 32 != 0) return TF_ESHAPE;
   if (B * nh * ((S + 127) / 128) > 0x7fffffff || S > (1 << 24)) return TF_EINVAL;
   if (sb % 8 || sh % 8 || ss % 8 || ss < hd) return TF_EALIGN;
   if (osb % 8 || osh % 8 || oss % 8 || oss < hd) return TF_EALIGN;

@@ -381,47 +381,18 @@ def _strided_ok(t):
     return t.stride(-1) == 1 and all(st % 8 == 0 for st in t.stride()[:-1]) and t.data_ptr() % 16 == 0
 
 
-def _pad_seq(t, pad):
-    """(B, nh, S, hd) -> contiguous (B, nh, S + pad, hd), zeros below."""
-    b, nh, s, hd = t.shape
-    out = torch.zeros((b, nh, s + pad, hd), dtype=t.dtype, device=t.device)
-    out[:, :, :s].copy_(t)
-    return out
-
-
-def _pad_bias(bias, need):
-    """A dense (nh, S', S') bias grown to S' >= need with zeros (what the extra rows and columns
-    hold never reaches a real query: their keys lie above its diagonal); slopes pass through."""
-    if bias is None or bias.ndim == 1 or bias.shape[1] >= need:
-        return bias
-    nh, sb, _ = bias.shape
-    out = torch.zeros((nh, need, need), dtype=bias.dtype, device=bias.device)
-    out[:, :sb, :sb].copy_(bias)
-    return out
-
-
 def flash_wrapper_fwd(q, k, v, bias=None, out=None):
     """Causal attention forward -> (out, lse).  ``bias``: None, a dense (nh, S', S') matrix, or
     the (nh,) float16 ALiBi slopes (the bias -slope_h * (i - j) is then computed in the kernel
     with the roundings of the reference's dense matrix).  ``out`` has q's strides unless a
     (B, nh, S, hd) view is passed in; ``lse`` is (B, nh, S) fp32 in the log2
     domain (the reference keeps fp16 m and l, kernels/attention.py:171-217 and
-    kernels/biased_attention.py:188-245); (B, nh, S + 32) when S is not a multiple of 64."""
+    kernels/biased_attention.py:188-245).  S % 32 == 0 for every head_dim (the reference: S % 64 == 0,
+    S % 32 == 0 at head_dim 128, kernels/attention.py:177-183)."""
     _check_attn(q, k, v, bias)
     b, nh, s, hd = q.shape
     if out is not None and (out.shape != q.shape or out.dtype != q.dtype or not _strided_ok(out)):
         raise ValueError("attention output buffer must match q in shape and dtype, with aligned strides")
-    if s % 64:
-        # head_dim 128 with S = 32 (mod 64), which the reference serves with 32-row blocks: the
-        # kernels work on 64-row blocks, so the sequence is continued by 32 rows of zeros.  Under
-        # the causal mask no real query sees an added key, and the added queries are dropped.  The
-        # log-sum-exp comes back for all S + 32 rows: the backward needs those of the added rows.
-        pad = 64 - s % 64
-        o_p, lse = flash_wrapper_fwd(_pad_seq(q, pad), _pad_seq(k, pad), _pad_seq(v, pad), _pad_bias(bias, s + pad))
-        if out is None:
-            out = torch.empty_strided(q.shape, q.stride(), dtype=q.dtype, device=q.device)
-        out.copy_(o_p[:, :, :s])
-        return out, lse
     q, k, v = _attn_layout(q, k, v)
     if out is None:
         out = torch.empty_strided(q.shape, q.stride(), dtype=q.dtype, device=q.device)
@@ -445,20 +416,6 @@ def flash_wrapper_bwd(grad_out, out, q, k, v, lse, bias=None, grads=None):
     into the three (B, nh, S, hd) views given as ``grads``); reference
     kernels/attention.py:550-607, kernels/biased_attention.py:598-660."""
     _check_attn(q, k, v, bias)
-    if q.shape[2] % 64:
-        # the zero-continued sequence of flash_wrapper_fwd: added rows carry zero output gradient,
-        # so they add nothing to dk, dv; their dq rows are dropped
-        s = q.shape[2]
-        pad = 64 - s % 64
-        if lse.shape[-1] != s + pad:
-            raise ValueError("lse must be the one flash_wrapper_fwd returned for this sequence")
-        got = flash_wrapper_bwd(_pad_seq(grad_out, pad), _pad_seq(out, pad), _pad_seq(q, pad), _pad_seq(k, pad),
-                                _pad_seq(v, pad), lse, _pad_bias(bias, s + pad))
-        if grads is None:
-            grads = tuple(torch.empty_strided(q.shape, q.stride(), dtype=q.dtype, device=q.device) for _ in range(3))
-        for dst, src in zip(grads, got):
-            dst.copy_(src[:, :, :s])
-        return grads
     q, k, v = _attn_layout(q, k, v)
     if not _strided_ok(out):
         out = out.contiguous()
