@@ -886,7 +886,9 @@ struct GemmGroup {
 };
 template <typename T, int BM, int BN, int BK, int WM, int WN, int WPE, bool A_KMAJOR, bool B_KMAJOR>
 __global__ __launch_bounds__(WM* WN * 64, WPE) void gemm_dma_group_kernel(GemmGroup g) {
-  const int pid = remap_xcd(blockIdx.x, g.first[g.count], g.p[0].xcds);
+  // (a group with a split tail keeps the ids as dealt, round-robin over the XCDs: whole tiles first, on every
+  // XCD alike, then the short slices of the tail -- the remap would hand all of the tail to the last XCDs)
+  const int pid = (g.p[0].flags & 1) ? (int)blockIdx.x : remap_xcd(blockIdx.x, g.first[g.count], g.p[0].xcds);
   int i = 0;
 #pragma unroll
   for (int k = 1; k < kMaxGroup; ++k)
@@ -1438,6 +1440,13 @@ struct GroupPlan {
   bool grouped;   // one launch for all problems (otherwise: one tf_gemm_out_chunked call each)
   int splits;
   int64_t need;   // workspace bytes
+  // Tiles that make whole rounds of workgroups plus a remainder: the last `cut_cols` tile columns of problem
+  // `cut_problem` (-1: none) become a member of the group of their own whose contraction is cut into
+  // `tail_splits` slices, so that the remainder fills one short round of all CUs instead of a whole round of
+  // a few (what the N-cut of a single product does for the LM-head weight gradient).
+  int cut_problem;
+  int cut_cols;
+  int tail_splits;
 };
 
 bool group_problem_ok(const tf_gemm_problem& q) {
@@ -1454,7 +1463,7 @@ bool group_problem_fast(const tf_gemm_problem& q) {
 }
 
 GroupPlan plan_group(int la, int lb, int count, const tf_gemm_problem* pr) {
-  GroupPlan gp = {false, 1, 0};
+  GroupPlan gp = {false, 1, 0, -1, 0, 1};
   bool fast = count >= 2 && count <= kMaxGroup && la == TF_OP_KMINOR && lb == TF_OP_KMINOR;
   const int64_t cus = device_shape().cus;
   int64_t tiles = 0, min_ksteps = INT64_MAX;
@@ -1479,6 +1488,41 @@ GroupPlan plan_group(int la, int lb, int count, const tf_gemm_problem* pr) {
     gp.splits = (int)splits;
     if (splits > 1)
       for (int i = 0; i < count; ++i) gp.need += splits * pr[i].M * pr[i].N * (int64_t)sizeof(float);
+    // More tiles than CUs and a remainder: look for a cut.  Costs in 64-wide contraction steps of a round of
+    // workgroups; the split tail pays its fp32 partials and the reduce pass (about six steps' worth).
+    bool same_k = true;
+    for (int i = 1; i < count; ++i) same_k = same_k && pr[i].K == pr[0].K;
+#ifdef TF_NO_GROUP_CUT
+    same_k = false;
+#endif
+    if (splits == 1 && tiles > cus && tiles % cus != 0 && same_k && count < kMaxGroup) {
+      const int64_t ksteps = pr[0].K / 64;
+      const int64_t rounds_whole = tiles / cus;
+      int64_t best = ((tiles + cus - 1) / cus) * ksteps * 9 / 10;  // a cut must win by a tenth
+      for (int i = 0; i < count; ++i) {
+        const bool unchunked = pr[i].chunk_n <= 0 || pr[i].chunk_n >= pr[i].N;
+        if (!unchunked || pr[i].M % 256 || pr[i].N % 256) continue;
+        const int64_t tm = pr[i].M / 256, tn = pr[i].N / 256;
+        for (int64_t c = 1; c < tn; ++c) {
+          const int64_t tail = c * tm;
+          if (tiles - tail > rounds_whole * cus) continue;  // the whole tiles must fit the whole rounds
+          int64_t s = cus / tail;
+          if (s > ksteps / 8) s = ksteps / 8;               // slices of at least 8 steps
+          if (s > 16) s = 16;
+          if (s < 2) break;
+          const int64_t per = (ksteps + s - 1) / s;
+          const int64_t cost = rounds_whole * ksteps + per + 6;
+          if (cost < best) {
+            best = cost;
+            gp.cut_problem = i;
+            gp.cut_cols = (int)c;
+            gp.tail_splits = (int)((ksteps + per - 1) / per);
+          }
+        }
+      }
+      if (gp.cut_problem >= 0)
+        gp.need = (int64_t)gp.tail_splits * pr[gp.cut_problem].M * gp.cut_cols * 256 * (int64_t)sizeof(float);
+    }
     return gp;
   }
   for (int i = 0; i < count; ++i) {
@@ -1514,12 +1558,40 @@ extern "C" int tf_gemm_group(void* stream, int dtype, int out_dtype, int layout_
     return TF_OK;
   }
   if (gp.need > 0 && !aligned16(workspace)) return TF_EALIGN;
+  // members of the launch: the problems as given, except that a cut problem keeps its leading columns and a
+  // further member takes its last tile columns with a split contraction
+  tf_gemm_problem mem[kMaxGroup];
+  int mem_splits[kMaxGroup];
+  int members = 0;
+  for (int i = 0; i < count; ++i) {
+    mem[members] = problems[i];
+    mem_splits[members] = gp.splits;
+    if (i == gp.cut_problem) mem[members].N -= (int64_t)gp.cut_cols * 256;
+    ++members;
+  }
+  if (gp.cut_problem >= 0) {
+    const tf_gemm_problem& q = problems[gp.cut_problem];
+    const int64_t n1 = q.N - (int64_t)gp.cut_cols * 256;
+    const int64_t osz = out_dtype == TF_F32 ? 4 : 2;
+    tf_gemm_problem t = q;
+    t.N = q.N - n1;
+    t.B = (const char*)q.B + n1 * 2;  // (K, N) row-major: the columns from n1 on
+    t.C = (char*)q.C + n1 * osz;
+    t.chunk_n = 0;
+    t.chunk_stride = 0;
+    mem[gp.cut_problem].chunk_n = 0;  // (only unchunked problems are cut)
+    mem[gp.cut_problem].chunk_stride = 0;
+    mem[members] = t;
+    mem_splits[members] = gp.tail_splits;
+    ++members;
+  }
   GemmGroup g;
-  g.count = count;
+  g.count = members;
   g.first[0] = 0;
   char* ws = (char*)workspace;
   for (int i = 0; i < kMaxGroup; ++i) {
-    const tf_gemm_problem& q = problems[i < count ? i : 0];
+    const tf_gemm_problem& q = mem[i < members ? i : 0];
+    const int want = mem_splits[i < members ? i : 0];
     GemmParams& p = g.p[i];
     const int64_t cn = (q.chunk_n <= 0 || q.chunk_n >= q.N) ? q.N : q.chunk_n;
     p.A = q.A; p.B = q.B; p.C = q.C; p.bias = nullptr; p.partial = (float*)ws;
@@ -1528,10 +1600,10 @@ extern "C" int tf_gemm_group(void* stream, int dtype, int out_dtype, int layout_
     p.relu = 0;
     p.tiles_m = (int)((q.M + 255) / 256); p.tiles_n = (int)((q.N + 255) / 256);
     const int64_t ksteps = q.K / 64;
-    const int64_t steps_per = (ksteps + gp.splits - 1) / gp.splits;
+    const int64_t steps_per = (ksteps + want - 1) / want;
     p.k_per_split = (int)(steps_per * 64);
     p.splits = (int)((ksteps + steps_per - 1) / steps_per);
-    p.flags = 0;
+    p.flags = gp.cut_problem >= 0 ? 1 : 0;
     p.xcds = device_shape().xcds;
     p.out_f32 = out_dtype == TF_F32 ? 1 : 0;
     p.mask = nullptr; p.ldmask = 0;
@@ -1539,9 +1611,9 @@ extern "C" int tf_gemm_group(void* stream, int dtype, int out_dtype, int layout_
     p.chunk_n = (int)cn;
     p.chunk_skip = (cn == q.N ? q.N : q.chunk_stride) - cn;
     p.alpha = nullptr;
-    if (i < count) {
+    if (i < members) {
       g.first[i + 1] = g.first[i] + p.tiles_m * p.tiles_n * p.splits;
-      if (p.splits > 1) ws += (int64_t)gp.splits * q.M * q.N * (int64_t)sizeof(float);
+      if (p.splits > 1) ws += (int64_t)want * q.M * q.N * (int64_t)sizeof(float);
     }
   }
   hipStream_t st = (hipStream_t)stream;
