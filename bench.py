@@ -436,6 +436,40 @@ def attention_probe(workload, dtype, device, iters=20):
             "tflops": round(flop / us / 1e6, 1)}
 
 
+def softmax_probe(device, iters=20):
+    """The row softmax kernels alone (tritonformer_amd.Softmax forward and backward), HIP events around `iters`
+    back-to-back calls: algorithmic bytes (forward: read x, write y; backward: read dy, y, write dx) per second
+    against the HBM peak, for 16-bit and fp32 rows of attention-score and vocabulary length."""
+    from tritonformer_amd import kernels as K
+
+    rows_out = []
+    for dt, name in ((torch.float16, "fp16"), (torch.bfloat16, "bf16"), (torch.float32, "fp32")):
+        for cols, rows in ((2048, 65536), (50304, 4096)):
+            es = 4 if dt == torch.float32 else 2
+            x = torch.randn(1, rows, cols, device=device).to(dt)
+            y = K.softmax_fwd(x)
+            dy = torch.randn_like(y)
+
+            def timed(fn):
+                for _ in range(2):
+                    fn()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(iters):
+                    fn()
+                e1.record()
+                torch.cuda.synchronize()
+                return e0.elapsed_time(e1) / iters * 1e3
+
+            for what, us, nbytes in (("forward", timed(lambda: K.softmax_fwd(x)), 2.0 * es * rows * cols),
+                                     ("backward", timed(lambda: K.softmax_bwd(dy, y)), 3.0 * es * rows * cols)):
+                gbs = nbytes / us / 1e3
+                rows_out.append({"pass": what, "dtype": name, "rows": rows, "cols": cols, "us": round(us, 1),
+                                 "GB/s": round(gbs, 1), "frac_of_hbm_peak": round(gbs / PEAK_HBM_GBS, 3)})
+            del x, y, dy
+    return {"probe": "row softmax forward / backward alone", "iters": iters, "peak_GB/s": PEAK_HBM_GBS, "results": rows_out}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -460,6 +494,9 @@ def main():
     ap.add_argument("--vendor-compare", metavar="FILE",
                     help="instead of the step: every dense product of the workload timed alone through this library and "
                          "through torch.matmul (the vendor BLAS library); writes a markdown table to FILE")
+    ap.add_argument("--softmax-probe", action="store_true",
+                    help="instead of the step: the row softmax kernels alone (16-bit and fp32 rows of 2048 and 50304 "
+                         "columns), GB/s against the HBM peak, one JSON line")
     ap.add_argument("--attention-probe", action="store_true",
                     help="instead of the step: the attention kernels of one layer of the workload alone, one JSON line")
     args = ap.parse_args()
@@ -476,6 +513,9 @@ def main():
         return
     if args.attention_probe:
         print(json.dumps(attention_probe(args.workload, dtype, device)))
+        return
+    if args.softmax_probe:
+        print(json.dumps(softmax_probe(device)))
         return
     if args.vendor_compare:
         print(json.dumps(vendor_compare(args.workload, dtype, device, args.vendor_compare)))

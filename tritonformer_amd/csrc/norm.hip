@@ -441,6 +441,126 @@ __global__ __launch_bounds__(256) void softmax_bwd_any(int64_t rows, int cols, c
 }
 
 // ---------------------------------------------------------------------------
+// Long rows (beyond the 512 chunks a single wave holds: vocabulary-sized rows): one workgroup of 16
+// waves per row, the row in registers as NV 16-byte chunks per thread (chunk c of thread t:
+// t + 1024 c), wave sums merged through LDS.  Every element is read once and written once, as in
+// the wave-per-row kernels.
+// ---------------------------------------------------------------------------
+constexpr int kLongRowThreads = 1024;
+// all-reduce of one value per thread over the workgroup; `slot` distinguishes consecutive uses
+template <bool MAX> __device__ __forceinline__ float block_reduce16(float v, float* red, int slot) {
+  v = MAX ? wave_max(v) : wave_sum(v);
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) red[slot * 16 + wave] = v;
+  __syncthreads();
+  float r = red[slot * 16];
+#pragma unroll
+  for (int w = 1; w < 16; ++w) r = MAX ? fmaxf(r, red[slot * 16 + w]) : r + red[slot * 16 + w];
+  return r;
+}
+
+template <typename T> __device__ __forceinline__ void chunk_floats(u32x4 raw, float (&v)[Chunk<T>::N]) {
+  if constexpr (sizeof(T) == 2) unpack8<T>(raw, v);
+  else {
+    const f32x4 f = __builtin_bit_cast(f32x4, raw);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = f[i];
+  }
+}
+// (exponentials of non-positive arguments: v_exp_f32 as it is, without the library wrapper's range
+// handling -- results below 2^-126 become zero, which is what they round to in the sum anyway)
+template <typename T, int NV>
+__global__ __launch_bounds__(kLongRowThreads) void softmax_fwd_long(int cols, const T* __restrict__ x, int64_t ldx,
+                                                                    T* __restrict__ y, int64_t ldy) {
+  constexpr int N = Chunk<T>::N;
+  __shared__ float red[32];
+  const int64_t row = blockIdx.x;
+  const int nchunk = cols / N;
+  const T* xr = x + row * ldx;
+  float v[NV][N];
+  float m = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = threadIdx.x + i * kLongRowThreads;
+    if (c < nchunk) {
+      chunk_floats<T>(ld16_stream(xr + c * N), v[i]);
+#pragma unroll
+      for (int e = 0; e < N; ++e) m = fmaxf(m, v[i][e]);
+    }
+  }
+  m = block_reduce16<true>(m, red, 0);
+  const float shift = -m * kLog2e;
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    if ((int)threadIdx.x + i * kLongRowThreads < nchunk) {
+#pragma unroll
+      for (int e = 0; e < N; ++e) { v[i][e] = __builtin_amdgcn_exp2f(__builtin_fmaf(v[i][e], kLog2e, shift)); s += v[i][e]; }
+    }
+  }
+  const float inv = 1.0f / block_reduce16<false>(s, red, 1);
+  T* yr = y + row * ldy;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = threadIdx.x + i * kLongRowThreads;
+    if (c < nchunk) {
+#pragma unroll
+      for (int e = 0; e < N; ++e) v[i][e] *= inv;
+      Chunk<T>::store(yr + c * N, v[i]);
+    }
+  }
+}
+
+// y and dy stay in registers as the raw 16-byte chunks (converted where they are used: as floats, 16-bit
+// rows would need twice the registers); with HOLD_DY false dy is read a second time instead (from the
+// cache: a row is a few hundred KB), for rows whose two operands do not fit the 128 registers of a thread.
+template <typename T, int NV, bool HOLD_DY>
+__global__ __launch_bounds__(kLongRowThreads) void softmax_bwd_long(int cols, const T* __restrict__ dy, int64_t lddy,
+                                                                    const T* __restrict__ y, int64_t ldy,
+                                                                    T* __restrict__ dx, int64_t lddx) {
+  constexpr int N = Chunk<T>::N;
+  __shared__ float red[16];
+  const int64_t row = blockIdx.x;
+  const int nchunk = cols / N;
+  u32x4 ry[NV], rg[HOLD_DY ? NV : 1];
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = threadIdx.x + i * kLongRowThreads;
+    if (c < nchunk) {
+      ry[i] = ld16_stream(y + row * ldy + c * N);
+      const u32x4 g = HOLD_DY ? ld16_stream(dy + row * lddy + c * N) : ld16(dy + row * lddy + c * N);
+      if (HOLD_DY) rg[i] = g;
+      float yv[N], gv[N];
+      chunk_floats<T>(ry[i], yv);
+      chunk_floats<T>(g, gv);
+#pragma unroll
+      for (int e = 0; e < N; ++e) s += yv[e] * gv[e];
+    }
+  }
+  s = block_reduce16<false>(s, red, 0);
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = threadIdx.x + i * kLongRowThreads;
+    if (c < nchunk) {
+      float yv[N], gv[N], o[N];
+      chunk_floats<T>(ry[i], yv);
+      chunk_floats<T>(HOLD_DY ? rg[i] : ld16(dy + row * lddy + c * N), gv);
+#pragma unroll
+      for (int e = 0; e < N; ++e) o[e] = yv[e] * (gv[e] - s);
+      Chunk<T>::store(dx + row * lddx + c * N, o);
+    }
+  }
+}
+// chunks per thread of the long-row kernels for a row of `nchunk` chunks (0: beyond them)
+template <typename T> static int pick_long_nv(int64_t nchunk) {
+  if (nchunk <= 4 * kLongRowThreads) return 4;
+  if (nchunk <= 8 * kLongRowThreads) return 8;
+  if (nchunk <= 16 * kLongRowThreads && sizeof(T) == 4) return 16;  // 65536 elements of either width
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
 // host dispatch
 // ---------------------------------------------------------------------------
 static int pick_nv(int64_t nchunk) {
@@ -531,7 +651,14 @@ static int softmax_fwd_launch(hipStream_t st, int64_t rows, int64_t cols, const 
     case 2: SM_FWD(2); break;
     case 4: SM_FWD(4); break;
     case 8: SM_FWD(8); break;
-    default: softmax_fwd_any<T><<<grid, block, 0, st>>>(rows, (int)cols, (const T*)x, ldx, (T*)y, ldy);
+    default: {
+      const int lnv = vec && rows <= 0x7fffffff ? pick_long_nv<T>(cols / Chunk<T>::N) : 0;
+      const dim3 lgrid((unsigned)rows), lblock(kLongRowThreads);
+      if (lnv == 4) softmax_fwd_long<T, 4><<<lgrid, lblock, 0, st>>>((int)cols, (const T*)x, ldx, (T*)y, ldy);
+      else if (lnv == 8) softmax_fwd_long<T, 8><<<lgrid, lblock, 0, st>>>((int)cols, (const T*)x, ldx, (T*)y, ldy);
+      else if (lnv == 16 && sizeof(T) == 4) softmax_fwd_long<float, 16><<<lgrid, lblock, 0, st>>>((int)cols, (const float*)x, ldx, (float*)y, ldy);
+      else softmax_fwd_any<T><<<grid, block, 0, st>>>(rows, (int)cols, (const T*)x, ldx, (T*)y, ldy);
+    }
   }
 #undef SM_FWD
   TF_CHECK_LAUNCH();
@@ -552,8 +679,17 @@ static int softmax_bwd_launch(hipStream_t st, int64_t rows, int64_t cols, const 
     case 2: SM_BWD(2); break;
     case 4: SM_BWD(4); break;
     case 8: SM_BWD(8); break;
-    default:
-      softmax_bwd_any<T><<<grid, block, 0, st>>>(rows, (int)cols, (const T*)dy, lddy, (const T*)y, ldy, (T*)dx, lddx);
+    default: {
+      const int lnv = vec && rows <= 0x7fffffff ? pick_long_nv<T>(cols / Chunk<T>::N) : 0;
+      const dim3 lgrid((unsigned)rows), lblock(kLongRowThreads);
+#define SM_BWD_LONG(TT, NV, HOLD) \
+  softmax_bwd_long<TT, NV, HOLD><<<lgrid, lblock, 0, st>>>((int)cols, (const TT*)dy, lddy, (const TT*)y, ldy, (TT*)dx, lddx)
+      if (lnv == 4) SM_BWD_LONG(T, 4, true);
+      else if (lnv == 8) SM_BWD_LONG(T, 8, true);
+      else if (lnv == 16 && sizeof(T) == 4) SM_BWD_LONG(float, 16, false);
+      else softmax_bwd_any<T><<<grid, block, 0, st>>>(rows, (int)cols, (const T*)dy, lddy, (const T*)y, ldy, (T*)dx, lddx);
+#undef SM_BWD_LONG
+    }
   }
 #undef SM_BWD
   TF_CHECK_LAUNCH();

@@ -18,6 +18,11 @@ template <> struct Chunk<float> {
 #pragma unroll
     for (int i = 0; i < 4; ++i) v[i] = r[i];
   }
+  static __device__ __forceinline__ void load_stream(const float* p, float (&v)[4]) {
+    f32x4 r = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = r[i];
+  }
   static __device__ __forceinline__ void store(float* p, const float (&v)[4]) {
     f32x4 r;
 #pragma unroll
