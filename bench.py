@@ -616,7 +616,15 @@ def main():
         # reference-named Functions only (LinearNoBias x 4 + LinearNoBiasReLU per block, CausalAttention,
         # LayerNorm, `residual + hidden`, nn.Embedding, logits + CrossEntropyLoss); headline protocol otherwise
         import tritonformer_amd.transformer as TM
-        flags = ("FUSE_QKV", "FUSE_MLP", "FUSE_ATTN_BLOCK", "FUSE_ADD_LN", "FUSE_EMBED", "FUSE_HEAD")
+        # the headline graph with every weight gradient launched inside its layer's backward (no queue across layers)
+        TM.DEFER_DW = False
+        try:
+            ms_i, loss_i = time_steps(model, tokens, k, w, dtype)
+        finally:
+            TM.DEFER_DW = True
+        out["weight_gradients_in_layer"] = {"ms_per_step": round(ms_i, 3), "steps": k,
+                                            "value": round(flops / (ms_i * 1e-3) / 1e12, 2), "loss": round(loss_i, 4)}
+        flags = ("FUSE_QKV", "FUSE_MLP", "FUSE_ATTN_BLOCK", "FUSE_ADD_LN", "FUSE_EMBED", "FUSE_HEAD", "DEFER_DW")
         saved = {n: getattr(TM, n) for n in flags}
         try:
             for n in flags:

@@ -143,14 +143,16 @@ int tf_gemm_scaled(void* stream, int dtype, int out_dtype, int layout_a, int lay
                    void* C, int64_t ldc, const float* alpha,
                    void* workspace, int64_t workspace_bytes);
 
-/* `count` (1..4) independent products of one dtype and one pair of operand layouts,
+/* `count` (1..8) independent products of one dtype and one pair of operand layouts,
  * no bias / ReLU / mask, each with the arguments of tf_gemm_out_chunked.  When every
  * problem meets the fast-path preconditions and both operands are TF_OP_KMINOR (the
  * weight-gradient form x^T . dy of tritonformer/linear.py:24-25), all of them run in
  * ONE launch: outputs with few tiles (two MLP weights: 64 tiles each) then fill the
  * GPU side by side, with half as many contraction slices and fp32 partials as two
- * launches would need.  Otherwise the problems run one after the other.  The results
- * do not depend on which of the two happens beyond the fp32 summation order. */
+ * launches would need; products whose tiles together make whole rounds of one workgroup
+ * per CU (the weight gradients of several layers, handed over together) run unsplit.
+ * Otherwise the problems run one after the other.  The results do not depend on which
+ * of the two happens beyond the fp32 summation order. */
 typedef struct tf_gemm_problem {
   int64_t M, N, K;
   const void* A; int64_t lda;

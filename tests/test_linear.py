@@ -411,13 +411,15 @@ def test_cast_pack_and_chunked_weight_gradient(dev):
         K.mm_dw(x, dy, chunks=5)
 
 
-@pytest.mark.parametrize("case", ["mlp-410m", "mlp-840m", "ragged", "chunked", "single"])
+@pytest.mark.parametrize("case", ["mlp-410m", "mlp-840m", "ragged", "chunked", "single", "eight"])
 def test_grouped_weight_gradients_equal_separate_products(case, dev):
     """mm_dw_group against one mm_dw per problem: same products, summed in fp32 (the
     contraction may be cut into a different number of slices), fp32 and fp16 outputs;
     'ragged' has extents the one-launch path cannot take and runs problem by problem;
     'mlp-840m' has 288 tiles, a round of workgroups and an eighth: the launch keeps whole tiles
-    for the round and splits the contraction of the last tile columns of one product."""
+    for the round and splits the contraction of the last tile columns of one product; 'eight' is the
+    form in which the weight gradients of several layers are handed over together: 256 tiles, one
+    round of workgroups, every contraction unsplit."""
     from tritonformer_amd import kernels as K
 
     g = torch.Generator().manual_seed(7)
@@ -425,24 +427,27 @@ def test_grouped_weight_gradients_equal_separate_products(case, dev):
               "mlp-840m": [((1, 4096, 1536), 6144), ((1, 4096, 6144), 1536)],
               "ragged": [((2, 77, 136), 72), ((2, 77, 72), 333)],
               "chunked": [((2, 512, 256), 768), ((2, 512, 256), 256), ((2, 512, 768), 256)],
-              "single": [((1, 640, 512), 512)]}[case]
+              "single": [((1, 640, 512), 512)],
+              "eight": [((1, 512, 1024), 3072), ((1, 512, 1024), 1024)] * 2
+                       + [((1, 512, 1024), 4096), ((1, 512, 4096), 1024)]
+                       + [((1, 512, 1024), 3072), ((1, 512, 1024), 1024)]}[case]
     pairs = [((torch.randn(*xs, generator=g)).half().to(dev), torch.randn(*xs[:-1], n, generator=g).half().to(dev))
              for xs, n in shapes]
-    chunks = [3, 1, 1] if case == "chunked" else [1] * len(pairs)
+    chunks = {"chunked": [3, 1, 1], "eight": [3, 1, 3, 1, 1, 1, 3, 1]}.get(case, [1] * len(pairs))
     for od in (torch.float32, None):
         outs = K.mm_dw_group(pairs, out_dtype=od, chunks=chunks)
         for (x, gr), ch, got in zip(pairs, chunks, outs):
             want = K.mm_dw(x, gr, out_dtype=od, chunks=ch)
             assert got.shape == want.shape and got.dtype == want.dtype and got.is_contiguous()
             assert rel_l2(got, want) < (1e-5 if od is torch.float32 else 1e-3)
-        if case.startswith("mlp") and od is torch.float32:   # and against the fp32 oracle
+        if (case.startswith("mlp") or case == "eight") and od is torch.float32:   # and against the fp32 oracle
             for (x, gr), got in zip(pairs, outs):
                 ref = x.float().cpu().reshape(-1, x.shape[-1]).T @ gr.float().cpu().reshape(-1, gr.shape[-1])
-                assert rel_l2(got, ref) < 1e-4
+                assert rel_l2(got.transpose(0, 1).reshape(ref.shape) if got.ndim == 3 else got, ref) < 1e-4
             again = K.mm_dw_group(pairs, out_dtype=od, chunks=chunks)   # fixed summation order: the same bits
             assert all(torch.equal(a, b) for a, b in zip(again, outs))
     with pytest.raises(ValueError):
-        K.mm_dw_group(pairs * 5)
+        K.mm_dw_group(pairs * 9)
 
 
 @pytest.mark.gpu

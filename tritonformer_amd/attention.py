@@ -5,6 +5,7 @@ from typing import Any, Tuple
 import torch
 from torch.autograd import Function
 
+from . import _deferred
 from ._amp import amp_bwd, amp_fwd, cached_conversion
 from .kernels import (
     cast_pack,
@@ -118,6 +119,10 @@ class AttentionBlock(Function):
         attn_bias = _bias_for(attn_bias, x.dtype)
         b, s, d = x.shape
         hd = d // num_heads
+        weights = (wq, wk, wv, wo)
+        same = all(w.dtype == wq.dtype for w in weights)
+        # the weights as the caller holds them: where their gradients go when they are deferred
+        ctx.defer_to = weights if _deferred.active() and same and _deferred.deferrable(weights) else None
         # the four (d, d) weights side by side in one 16-bit (d, 4d) matrix, one conversion kernel;
         # the GEMMs take its first three column blocks and its last one as strided operands
         packed = cached_conversion([wq, wk, wv, wo], x.dtype, cast_pack)
@@ -143,6 +148,12 @@ class AttentionBlock(Function):
         grads = tuple(dqkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
         flash_wrapper_bwd(d_attn, attn.view(b, s, nh, hd).permute(0, 2, 1, 3), q, k, v, lse, attn_bias, grads=grads)
         dqkv = dqkv.view(b, s, 3 * nh * hd)
+        if ctx.defer_to is not None:
+            # launched later, together with those of other layers, in whole rounds of workgroups
+            _deferred.submit([(x, dqkv, 3, ctx.defer_to[:3], ctx.weight_dtype),
+                              (attn, grad_output, 1, ctx.defer_to[3:], ctx.weight_dtype)])
+            grad_x = mm(dqkv, w_qkv.T) if ctx.needs_input_grad[0] else None
+            return grad_x, None, None, None, None, None, None
         # weight gradients first, the input gradient (what the next kernel reads) last
         d_wqkv, d_wo = mm_dw_group([(x, dqkv), (attn, grad_output)], out_dtype=ctx.weight_dtype, chunks=[3, 1])
         grad_x = mm(dqkv, w_qkv.T) if ctx.needs_input_grad[0] else None

@@ -875,10 +875,10 @@ __global__ __launch_bounds__(WM* WN * 64, WPE) void gemm_dma_kernel(GemmParams p
   gemm_dma_body<T, BM, BN, BK, WM, WN, A_KMAJOR, B_KMAJOR>(p, pid);
 }
 
-// Up to four independent products of one operand layout in ONE launch: workgroup ids
+// Up to eight independent products of one operand layout in ONE launch: workgroup ids
 // [first[i], first[i+1]) belong to problem i.  Used for weight gradients, whose output has
 // few tiles: side by side they fill the chip with fewer, longer contraction slices.
-constexpr int kMaxGroup = 4;
+constexpr int kMaxGroup = 8;
 struct GemmGroup {
   GemmParams p[kMaxGroup];
   int first[kMaxGroup + 1];

@@ -3,6 +3,7 @@ the reference's tritonformer/linear.py.  Weight layout is (in, out): y = x @ W."
 import torch
 from torch.autograd import Function
 
+from . import _deferred
 from ._amp import amp_bwd, amp_fwd, cached_conversion
 from .kernels import (cast_pack, gemm, gemm_relu_bits, mask_grad, mm, mm_dw, mm_dw_group, mm_masked_bits,
                       unbroadcast_leading)
@@ -121,6 +122,8 @@ class MLPReLU(Function):
     @staticmethod
     @amp_fwd(keep=(1, 3))
     def forward(ctx, input, w1, b1, w2, b2):
+        # the weights as the caller holds them: where their gradients go when they are deferred
+        ctx.defer_to = (w1, w2) if _deferred.active() and GROUP_DW and _deferred.deferrable((w1, w2)) else None
         if ctx.amp_active and (w1.dtype != input.dtype or w2.dtype != input.dtype):
             # what autocast's cast of the two weights does -- as ONE conversion kernel over both when
             # they are stored alike (two matrices of d*f elements each seen as two rows)
@@ -155,7 +158,13 @@ class MLPReLU(Function):
         grad_b2 = _bias_grad(ctx, grad_output, 4) if ctx.has_bias[1] else None
         # the weight gradients first, the input gradient last: what the next kernel of the backward
         # pass reads is then what was written last (0.1 ms per step of the 410M model)
-        if GROUP_DW and ctx.arg_dtypes[1] == ctx.arg_dtypes[3]:
+        if ctx.defer_to is not None and ctx.arg_dtypes[1] == ctx.arg_dtypes[3]:
+            # launched later, together with those of other layers, in whole rounds of workgroups
+            master = f32 if ctx.arg_dtypes[1] == f32 else None
+            _deferred.submit([(input, grad_hidden, 1, ctx.defer_to[:1], master),
+                              (hidden, grad_output, 1, ctx.defer_to[1:], master)])
+            grad_w1 = grad_w2 = None
+        elif GROUP_DW and ctx.arg_dtypes[1] == ctx.arg_dtypes[3]:
             # both weight gradients side by side in one launch
             grad_w1, grad_w2 = mm_dw_group([(input, grad_hidden), (hidden, grad_output)],
                                            out_dtype=f32 if ctx.arg_dtypes[1] == f32 else None)
