@@ -240,6 +240,24 @@ int tf_layernorm_bwd(void* stream, int dtype, int param_dtype, int64_t rows, int
                      float* partial, int64_t partial_bytes);
 int64_t tf_layernorm_bwd_partial_bytes(int64_t rows, int64_t d);
 
+/* The second stage by itself, for the LayerNorms of a whole backward pass at once.
+ * tf_layernorm_bwd / tf_add_layernorm_bwd called with dgamma = dbeta = NULL write dx and
+ * leave the column sums of their row blocks in `partial`: tf_layernorm_bwd_parts(rows)
+ * rows of 2*d fp32 values (d of dgamma, then d of dbeta).  tf_layernorm_param_grads sums
+ * the rows of `count` such buffers (any count; one launch per 64) in the order the
+ * one-call form sums them -- the same bits -- into dgamma / dbeta of `param_dtype`.
+ * Stands where the reference launches its reductions.py second stage once per LayerNorm
+ * (kernels/layernorm.py:226-259). */
+typedef struct tf_ln_param_grads {
+  const float* partial;
+  int64_t parts;
+  void* dgamma;
+  void* dbeta;
+} tf_ln_param_grads;
+int64_t tf_layernorm_bwd_parts(int64_t rows);
+int tf_layernorm_param_grads(void* stream, int param_dtype, int64_t d, int count,
+                             const tf_ln_param_grads* items);
+
 /* Residual addition fused into the LayerNorm that follows it:
  *   sum = x + res (rounded to `dtype`, written out),  y = layernorm(sum).
  * One kernel for the reference model's `hidden_states = residual + hidden_states`

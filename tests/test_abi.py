@@ -232,6 +232,18 @@ def test_row_kernels_reject_bad_arguments():
     assert lib.tf_layernorm_bwd(None, 0, 0, 4, 64, FAKE, 64, FAKE, 64, FAKE, FAKE, FAKE, FAKE, 64, FAKE, FAKE,
                                 None, 0) == -5
     assert lib.tf_layernorm_bwd_partial_bytes(8192, 1024) == 512 * 2 * 1024 * 4
+    # the second stage by itself: dgamma and dbeta are given together or not at all; partial rows as the row pass cuts them
+    assert lib.tf_layernorm_bwd(None, 0, 0, 4, 64, FAKE, 64, FAKE, 64, FAKE, FAKE, FAKE, FAKE, 64, FAKE, None,
+                                FAKE, 1 << 20) == -1
+    assert lib.tf_layernorm_bwd(None, 0, 0, 4, 64, FAKE, 64, FAKE, 64, FAKE, FAKE, FAKE, FAKE, 64, None, None,
+                                None, 0) == -5
+    assert lib.tf_layernorm_bwd_parts(8192) == 512 and lib.tf_layernorm_bwd_parts(5) == 2 and lib.tf_layernorm_bwd_parts(0) == 0
+    item = (_lib.LnParamGrads * 2)(_lib.LnParamGrads(FAKE, 512, FAKE, FAKE), _lib.LnParamGrads(FAKE, 513, FAKE, FAKE))
+    assert lib.tf_layernorm_param_grads(None, 2, 1024, 0, None) == 0            # nothing to do
+    assert lib.tf_layernorm_param_grads(None, 2, 1024, 1, None) == -1
+    assert lib.tf_layernorm_param_grads(None, 2, 1024, 2, item) == -1           # more partial rows than a row pass writes
+    assert lib.tf_layernorm_param_grads(None, 3, 1024, 1, item) == -2
+    assert lib.tf_layernorm_param_grads(None, 2, 0, 1, item) == -1
     # fused residual add: missing summand / sum buffer, short leading dimension, missing workspace
     assert lib.tf_add_layernorm_fwd(None, 0, 0, 4, 64, FAKE, 64, None, 64, FAKE, 64, FAKE, FAKE, 1e-5, FAKE, 64, FAKE,
                                     FAKE) == -1

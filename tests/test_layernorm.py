@@ -162,3 +162,38 @@ def test_add_layernorm_unused_outputs(dev):
     assert torch.equal(x.grad, dy) and torch.equal(br.grad, dy) and gamma.grad is None
     with pytest.raises(ValueError):
         T.add_layer_norm.apply(x, br[:, :5], gamma, beta, 1e-5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("pdtype", [torch.float32, torch.float16])
+def test_param_grads_of_many_layernorms_in_one_launch(pdtype, dev):
+    """Row passes that leave their partial sums in place, then ONE second stage for all of them
+    (tf_layernorm_param_grads, 70 LayerNorms: a launch of 64 and one of 6) against the one-call
+    form that the reference's structure has (kernels/layernorm.py:226-259): same dx, same bits in
+    dgamma / dbeta; plain and residual-adding row passes, different row counts."""
+    from tritonformer_amd import kernels as K
+
+    g = torch.Generator().manual_seed(5)
+    d = 256
+    want, partials = [], []
+    for i in range(70):
+        rows = (3, 64 + 7 * i)
+        x = torch.randn(*rows, d, generator=g).half().to(dev)
+        dy = torch.randn(*rows, d, generator=g).half().to(dev)
+        gamma = torch.randn(d, generator=g).to(pdtype).to(dev)
+        mean = x.float().mean(-1).reshape(-1)
+        rstd = (x.float().var(-1, unbiased=False) + 1e-5).rsqrt().reshape(-1)
+        if i % 2:
+            ds = torch.randn(*rows, d, generator=g).half().to(dev)
+            dx, da, db = K.add_layernorm_bwd(dy, ds, x, gamma, mean, rstd)
+            dx2, part = K.add_layernorm_bwd(dy, ds, x, gamma, mean, rstd, leave_partials=True)
+        else:
+            dx, da, db = K.layernorm_bwd(dy, x, gamma, mean, rstd)
+            dx2, part = K.layernorm_bwd(dy, x, gamma, mean, rstd, leave_partials=True)
+        assert torch.equal(dx, dx2)
+        want.append((da, db))
+        partials.append(part)
+    out = K.layernorm_param_grads(partials, d, pdtype)
+    assert out.shape == (70, 2, d) and out.dtype == pdtype
+    for i, (da, db) in enumerate(want):
+        assert torch.equal(out[i, 0], da) and torch.equal(out[i, 1], db), i

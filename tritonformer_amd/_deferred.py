@@ -1,4 +1,4 @@
-"""Weight gradients of the transformer blocks, launched in whole rounds of workgroups.
+"""Parameter gradients of the transformer blocks, launched when it suits the GPU rather than the graph.
 
 A weight gradient dW = X^T dY is needed by nobody until the backward pass ends, and the output of one
 such product has few 256x256 tiles (16 to 64 per weight of the 410M model on 256 CUs): launched where
@@ -11,12 +11,16 @@ engine finishes the pass.  The gradients are complete, on the stream the pass ra
 instead of through the Function's return value: a weight that is not a leaf, or carries hooks, is not
 deferred, and ``torch.autograd.grad`` with respect to such a weight must run with deferral off
 (it reports the weight as unused otherwise).
+
+The LayerNorms of the model use the same queue for the second stage of their gamma / beta gradients: the
+row pass leaves the column sums of its row blocks in place, and one launch at the end of the pass sums
+those of every LayerNorm (the reference launches that stage once per LayerNorm, kernels/layernorm.py:226-259).
 """
 import contextlib
 
 import torch
 
-from .kernels import mm_dw_group
+from .kernels import layernorm_param_grads, mm_dw_group
 
 # products per launch (the grouped GEMM entry point takes up to eight)
 _MAX_GROUP = 8
@@ -27,6 +31,7 @@ _MAX_PENDING = 12
 
 _enabled = False
 _pending = []
+_pending_ln = []
 _task = None
 _cus = {}
 
@@ -124,28 +129,59 @@ def _drain(final):
         _launch(items)
 
 
+def _finish_ln():
+    # one launch per kind (width, parameter dtype, device) -- one kind in a model
+    kinds = {}
+    for partial, d, params in _pending_ln:
+        kinds.setdefault((d, params[0].dtype, partial[0].device), []).append((partial, params))
+    with torch.no_grad():
+        for (d, dtype, _), members in kinds.items():
+            out = layernorm_param_grads([m[0] for m in members], d, dtype)
+            for i, (_, params) in enumerate(members):
+                for j, p in enumerate(params):
+                    if p.grad is None:
+                        p.grad = out[i, j]
+                    else:
+                        p.grad.add_(out[i, j])
+
+
 def _finish():
     global _task
     _task = None
     try:
         _drain(final=True)
+        if _pending_ln:
+            _finish_ln()
     finally:
         _pending.clear()
+        _pending_ln.clear()
+
+
+def _join_pass():
+    global _task
+    task = torch._C._current_graph_task_id()
+    if task < 0:
+        raise RuntimeError("deferred parameter gradients are submitted from inside a backward pass")
+    if task != _task:
+        # first submission of this pass (what an earlier pass that raised left behind is dropped)
+        _pending.clear()
+        _pending_ln.clear()
+        _task = task
+        torch.autograd.Variable._execution_engine.queue_callback(_finish)
+
+
+def submit_layernorm(partial, d, params):
+    """``partial``: what layernorm_bwd(..., leave_partials=True) returned beside dx; ``params`` = (gamma, beta)
+    of width ``d``, whose ``.grad`` receive the sums when the pass ends."""
+    _join_pass()
+    _pending_ln.append((partial, d, tuple(params)))
 
 
 def submit(products):
     """``products``: (x, grad, chunks, params, out_dtype) -- dW = x^T grad in ``out_dtype`` (None: the
     operands'), cut into ``chunks`` equal column blocks, block j added to ``params[j].grad``.  Call from
     inside a backward pass only."""
-    global _task
-    task = torch._C._current_graph_task_id()
-    if task < 0:
-        raise RuntimeError("deferred weight gradients are submitted from inside a backward pass")
-    if task != _task:
-        # first submission of this pass (what an earlier pass that raised left behind is dropped)
-        _pending.clear()
-        _task = task
-        torch.autograd.Variable._execution_engine.queue_callback(_finish)
+    _join_pass()
     for x, grad, chunks, params, out_dtype in products:
         _pending.append(_Product(x, grad, chunks, tuple(params), out_dtype))
     _drain(final=False)

@@ -51,6 +51,8 @@ SIGNATURES = {
     "tf_layernorm_bwd": (_i, [_vp, _i, _i, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp,
                               _i64]),
     "tf_layernorm_bwd_partial_bytes": (_i64, [_i64, _i64]),
+    "tf_layernorm_bwd_parts": (_i64, [_i64]),
+    "tf_layernorm_param_grads": (_i, [_vp, _i, _i64, _i, _vp]),
     "tf_add_layernorm_fwd": (_i, [_vp, _i, _i, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _f, _vp, _i64,
                                   _vp, _vp]),
     "tf_add_layernorm_bwd": (_i, [_vp, _i, _i, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64,
@@ -89,6 +91,11 @@ class GemmProblem(ctypes.Structure):
     """`tf_gemm_problem` of include/tritonformer_amd.h."""
     _fields_ = [("M", _i64), ("N", _i64), ("K", _i64), ("A", _vp), ("lda", _i64), ("B", _vp), ("ldb", _i64),
                 ("C", _vp), ("ldc", _i64), ("chunk_n", _i64), ("chunk_stride", _i64)]
+
+
+class LnParamGrads(ctypes.Structure):
+    """`tf_ln_param_grads` of include/tritonformer_amd.h."""
+    _fields_ = [("partial", _vp), ("parts", _i64), ("dgamma", _vp), ("dbeta", _vp)]
 
 
 DIAG_LIB_PATH = os.path.join(_HERE, "libtritonformer_amd_diag.so")

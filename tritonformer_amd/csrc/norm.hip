@@ -330,6 +330,46 @@ __global__ __launch_bounds__(256) void ln_bwd_reduce(int nparts, int d, const fl
   }
 }
 
+// The same second stage for the partial sums of several LayerNorms in one launch (blockIdx.y = LayerNorm):
+// the parameter gradients of a whole backward pass, whose partial sums were left in place by the row passes.
+constexpr int kLnReduceBatch = 64;
+struct LnReduceItem {
+  const float* partial;
+  void* dgamma;
+  void* dbeta;
+  int parts;
+};
+struct LnReduceBatch { LnReduceItem it[kLnReduceBatch]; };
+template <typename T>
+__global__ __launch_bounds__(256) void ln_bwd_reduce_batch(LnReduceBatch batch, int d) {
+  __shared__ float red[16][17];
+  const LnReduceItem r = batch.it[blockIdx.y];
+  const int cl = threadIdx.x & 15, slice = threadIdx.x >> 4;
+  const int col = blockIdx.x * 16 + cl;  // 0 .. 2d-1
+  float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+  if (col < 2 * d) {
+    const float* src = r.partial + col;
+    const int64_t ld = 2 * (int64_t)d;
+    int p = slice;
+    for (; p + 48 < r.parts; p += 64) {
+      a0 += src[(int64_t)p * ld];
+      a1 += src[(int64_t)(p + 16) * ld];
+      a2 += src[(int64_t)(p + 32) * ld];
+      a3 += src[(int64_t)(p + 48) * ld];
+    }
+    for (; p < r.parts; p += 16) a0 += src[(int64_t)p * ld];
+  }
+  red[slice][cl] = (a0 + a1) + (a2 + a3);
+  __syncthreads();
+  if (slice == 0 && col < 2 * d) {
+    float s = 0.f;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) s += red[k][cl];
+    if (col < d) ((T*)r.dgamma)[col] = (T)s;
+    else ((T*)r.dbeta)[col - d] = (T)s;
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Softmax (T = f16 / bf16 / float).  NV chunks of Chunk<T>::N elements per lane.
 // ---------------------------------------------------------------------------
@@ -634,6 +674,7 @@ static int ln_bwd_launch(hipStream_t st, int64_t rows, int64_t d, const void* dy
   }
 #undef LN_BWD
   TF_CHECK_LAUNCH();
+  if (!dgamma) return TF_OK;  // the partial sums stay where they are, for tf_layernorm_param_grads
   ln_bwd_reduce<TP><<<dim3(ceil_div(2 * d, 16)), dim3(256), 0, st>>>(parts, (int)d, partial, (TP*)dgamma, (TP*)dbeta);
   TF_CHECK_LAUNCH();
   return TF_OK;
@@ -747,7 +788,7 @@ static int ln_bwd_entry(void* stream, int dtype, int param_dtype, int64_t rows, 
                         int64_t lddy, const void* dsum, int64_t lddsum, const void* x, int64_t ldx,
                         const void* gamma, const float* mean, const float* rstd, void* dx, int64_t lddx,
                         void* dgamma, void* dbeta, float* partial, int64_t partial_bytes) {
-  if (!dy || !x || !gamma || !mean || !rstd || !dx || !dgamma || !dbeta) return TF_EINVAL;
+  if (!dy || !x || !gamma || !mean || !rstd || !dx || (dgamma == nullptr) != (dbeta == nullptr)) return TF_EINVAL;
   if (ADD && (!dsum || lddsum < d)) return TF_EINVAL;
   if (bad_rows(rows, d, ldx) || lddy < d || lddx < d || rows == 0) return TF_EINVAL;
   if (!partial || partial_bytes < tf_layernorm_bwd_partial_bytes(rows, d)) return TF_EWORKSPACE;
@@ -776,6 +817,30 @@ extern "C" int tf_add_layernorm_bwd(void* stream, int dtype, int param_dtype, in
                                     void* dgamma, void* dbeta, float* partial, int64_t partial_bytes) {
   return ln_bwd_entry<true>(stream, dtype, param_dtype, rows, d, dy, lddy, dsum, lddsum, x, ldx, gamma, mean, rstd, dx,
                             lddx, dgamma, dbeta, partial, partial_bytes);
+}
+
+extern "C" int64_t tf_layernorm_bwd_parts(int64_t rows) { return rows > 0 ? ln_bwd_parts(rows) : 0; }
+
+extern "C" int tf_layernorm_param_grads(void* stream, int param_dtype, int64_t d, int count,
+                                        const tf_ln_param_grads* items) {
+  if (count < 0 || d <= 0 || d > 0x3fffffff || (count > 0 && !items)) return TF_EINVAL;
+  if (param_dtype != TF_F16 && param_dtype != TF_BF16 && param_dtype != TF_F32) return TF_EDTYPE;
+  for (int i = 0; i < count; ++i)
+    if (!items[i].partial || !items[i].dgamma || !items[i].dbeta || items[i].parts < 1 || items[i].parts > 512)
+      return TF_EINVAL;
+  hipStream_t st = (hipStream_t)stream;
+  for (int base = 0; base < count; base += kLnReduceBatch) {
+    const int n = count - base < kLnReduceBatch ? count - base : kLnReduceBatch;
+    LnReduceBatch b = {};
+    for (int i = 0; i < n; ++i)
+      b.it[i] = {items[base + i].partial, items[base + i].dgamma, items[base + i].dbeta, (int)items[base + i].parts};
+    const dim3 grid((unsigned)ceil_div(2 * d, 16), (unsigned)n), block(256);
+    if (param_dtype == TF_F32) ln_bwd_reduce_batch<float><<<grid, block, 0, st>>>(b, (int)d);
+    else if (param_dtype == TF_F16) ln_bwd_reduce_batch<f16><<<grid, block, 0, st>>>(b, (int)d);
+    else ln_bwd_reduce_batch<bf16><<<grid, block, 0, st>>>(b, (int)d);
+    TF_CHECK_LAUNCH();
+  }
+  return TF_OK;
 }
 
 extern "C" int tf_softmax_fwd(void* stream, int dtype, int64_t rows, int64_t cols, const void* x, int64_t ldx,

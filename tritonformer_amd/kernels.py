@@ -483,22 +483,45 @@ def layernorm_fwd(x, alpha, beta, eps):
     return y, mean, rstd
 
 
-def layernorm_bwd(grad_out, x, alpha, mean, rstd):
+def layernorm_bwd(grad_out, x, alpha, mean, rstd, leave_partials=False):
     """-> (dx, dalpha, dbeta); reference dx_layernorm (kernels/layernorm.py:140-162)
-    and layernorm_da_db (kernels/layernorm.py:226-259) in one pass."""
+    and layernorm_da_db (kernels/layernorm.py:226-259) in one pass.  With ``leave_partials``
+    -> (dx, partial): the column sums of the row blocks as they are, for layernorm_param_grads."""
     lib = load()
     x2, rows, d = _rows2d(x)
     g2, _, _ = _rows2d(grad_out)
     dx = torch.empty(x.shape, dtype=x.dtype, device=x.device)
-    da = torch.empty((d,), dtype=alpha.dtype, device=x.device)
-    db = torch.empty((d,), dtype=alpha.dtype, device=x.device)
+    da = db = None
+    if not leave_partials:
+        da = torch.empty((d,), dtype=alpha.dtype, device=x.device)
+        db = torch.empty((d,), dtype=alpha.dtype, device=x.device)
     pb = lib.tf_layernorm_bwd_partial_bytes(rows, d)
     part = torch.empty(pb, dtype=torch.uint8, device=x.device)
     check(lib.tf_layernorm_bwd(stream_ptr(), dtype_code(x.dtype), dtype_code(alpha.dtype), rows, d, g2.data_ptr(), d,
                                x2.data_ptr(), d,
                                alpha.contiguous().data_ptr(), mean.data_ptr(), rstd.data_ptr(), dx.data_ptr(), d,
-                               da.data_ptr(), db.data_ptr(), part.data_ptr(), pb))
+                               None if da is None else da.data_ptr(), None if db is None else db.data_ptr(),
+                               part.data_ptr(), pb))
+    if leave_partials:
+        return dx, (part, lib.tf_layernorm_bwd_parts(rows))
     return dx, da, db
+
+
+def layernorm_param_grads(partials, d, dtype):
+    """``partials``: (buffer, parts) pairs that layernorm_bwd / add_layernorm_bwd left behind.  -> a
+    (len(partials), 2, d) tensor of ``dtype``: [i, 0] = dgamma and [i, 1] = dbeta of the i-th LayerNorm,
+    all of them summed by one launch (per 64)."""
+    lib = load()
+    n = len(partials)
+    device = partials[0][0].device
+    out = torch.empty((n, 2, d), dtype=dtype, device=device)
+    items = (_lib.LnParamGrads * n)()
+    step = 2 * d * out.element_size()
+    for i, (buf, parts) in enumerate(partials):
+        require_cuda(buf)
+        items[i] = _lib.LnParamGrads(buf.data_ptr(), parts, out.data_ptr() + i * step, out.data_ptr() + i * step + step // 2)
+    check(lib.tf_layernorm_param_grads(stream_ptr(), dtype_code(dtype), d, n, items))
+    return out
 
 
 def add_layernorm_fwd(x, res, alpha, beta, eps):
@@ -523,22 +546,28 @@ def add_layernorm_fwd(x, res, alpha, beta, eps):
     return total, y, mean, rstd
 
 
-def add_layernorm_bwd(grad_out, grad_sum, total, alpha, mean, rstd):
+def add_layernorm_bwd(grad_out, grad_sum, total, alpha, mean, rstd, leave_partials=False):
     """-> (dx, dalpha, dbeta): dx = layernorm backward of grad_out at the saved sum, plus
-    grad_sum (the gradient of the sum arriving along the residual stream)."""
+    grad_sum (the gradient of the sum arriving along the residual stream).  ``leave_partials`` as in
+    layernorm_bwd."""
     lib = load()
     x2, rows, d = _rows2d(total)
     g2, _, _ = _rows2d(grad_out)
     s2, _, _ = _rows2d(grad_sum)
     dx = torch.empty(total.shape, dtype=total.dtype, device=total.device)
-    da = torch.empty((d,), dtype=alpha.dtype, device=total.device)
-    db = torch.empty((d,), dtype=alpha.dtype, device=total.device)
+    da = db = None
+    if not leave_partials:
+        da = torch.empty((d,), dtype=alpha.dtype, device=total.device)
+        db = torch.empty((d,), dtype=alpha.dtype, device=total.device)
     pb = lib.tf_layernorm_bwd_partial_bytes(rows, d)
     part = torch.empty(pb, dtype=torch.uint8, device=total.device)
     check(lib.tf_add_layernorm_bwd(stream_ptr(), dtype_code(total.dtype), dtype_code(alpha.dtype), rows, d,
                                    g2.data_ptr(), d, s2.data_ptr(), d, x2.data_ptr(), d,
                                    alpha.contiguous().data_ptr(), mean.data_ptr(), rstd.data_ptr(), dx.data_ptr(), d,
-                                   da.data_ptr(), db.data_ptr(), part.data_ptr(), pb))
+                                   None if da is None else da.data_ptr(), None if db is None else db.data_ptr(),
+                                   part.data_ptr(), pb))
+    if leave_partials:
+        return dx, (part, lib.tf_layernorm_bwd_parts(rows))
     return dx, da, db
 
 
