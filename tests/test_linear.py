@@ -451,12 +451,14 @@ def test_grouped_weight_gradients_equal_separate_products(case, dev):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("dims", [(2, 128, 256, 1024), (1, 384, 128, 320)])
+@pytest.mark.parametrize("dims", [(2, 128, 256, 1024), (1, 384, 128, 320), (1, 4096, 1536, 6144)])
 @pytest.mark.parametrize("use_bias", [False, True])
 def test_relu_sign_bits_equal_the_activation_mask(dims, use_bias, dev):
     """gemm_relu_bits returns relu(x W + b) bit-identical to the plain ReLU GEMM, and one bit per
     element that says where it is positive (bit n % 8 of byte n / 8); the masked product taken
-    from those bits equals the one that reads the activation (kernels/activation.py:27-44)."""
+    from those bits equals the one that reads the activation (kernels/activation.py:27-44).
+    The last case has a round and a half of 256x256 tiles: both products are cut into whole rounds
+    and a remainder, each part with its share of the bit rows."""
     import numpy as np
     from tritonformer_amd import kernels as K
 

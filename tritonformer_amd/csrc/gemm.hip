@@ -1243,8 +1243,9 @@ static int64_t tail_columns(int64_t M, int64_t N, int64_t K, bool vec, bool allo
 // together are cheaper than the best single launch (q/k/v projection 8192 x 3072 x 1024: one
 // round of 256x256 tiles + 1024 columns of 128x128 tiles, 0.2 ms per training step less than
 // three rounds of 128x128 tiles).
-static int64_t round_cut_columns(int64_t M, int64_t N, int64_t K, bool vec, bool allow_split, const GemmForce& force) {
-  if (!allow_split || force.cfg >= 0 || force.splits > 0 || !(vec && K % 64 == 0) || (force.flags & 64)) return 0;
+static int64_t round_cut_columns(int64_t M, int64_t N, int64_t K, bool vec, bool allow_split, const GemmForce& force,
+                                 bool allow_cut) {
+  if (!allow_cut || force.cfg >= 0 || force.splits > 0 || !(vec && K % 64 == 0) || (force.flags & 64)) return 0;
   const int64_t cus = device_shape().cus;
   double uncut, whole, rest;
   (void)make_plan(M, N, K, vec, allow_split, &uncut);
@@ -1274,7 +1275,7 @@ extern "C" int64_t tf_gemm_workspace_bytes(int layout_a, int layout_b, int64_t M
   for (int vec = 0; vec < 2; ++vec) {
     int64_t n = single_need(M, N, K, vec != 0);
     int64_t tail = tail_columns(M, N, K, vec != 0, true, kNoForce);
-    if (tail == 0) tail = round_cut_columns(M, N, K, vec != 0, true, kNoForce);
+    if (tail == 0) tail = round_cut_columns(M, N, K, vec != 0, true, kNoForce, true);
     if (tail > 0) {
       const int64_t n1 = single_need(M, N - tail, K, vec != 0), n2 = single_need(M, tail, K, vec != 0);
       if (n1 > n) n = n1;
@@ -1333,20 +1334,30 @@ static int gemm_entry(void* stream, int dtype, int out_dtype, int layout_a, int 
   const bool vec = aligned16(A) && aligned16(B) && aligned16(C) && (!bias || aligned16(bias)) && a_contig % 8 == 0 &&
                    b_contig % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 && N % 8 == 0 && ldc % 8 == 0 &&
                    (!mask_act || (aligned16(mask_act) && ld_mask % 8 == 0));
-  if (chunk_n == N && !signs) {
-    int64_t tail = tail_columns(M, N, K, vec, mask_act == nullptr, force);
-    if (tail == 0) tail = round_cut_columns(M, N, K, vec, mask_act == nullptr, force);
+  if (chunk_n == N) {
+    // (a launch with sign bits takes no split contraction: its cut is the one into unsplit products, and only
+    // where the bits of both parts are served -- a cut at a multiple of 256 columns keeps whole bytes and the
+    // 16-byte pieces of the bit rows)
+    const bool may_split = mask_act == nullptr && !signs;
+    int64_t tail = signs ? 0 : tail_columns(M, N, K, vec, may_split, force);
+    if (tail == 0) tail = round_cut_columns(M, N, K, vec, may_split, force, mask_act == nullptr);
+    if (tail > 0 && signs) {
+      const GemmPlan p1 = make_plan(M, N - tail, K, vec, false, nullptr, force), p2 = make_plan(M, tail, K, vec, false, nullptr, force);
+      if (!(kCfgs[p1.cfg].dma && kCfgs[p2.cfg].dma && K % p1.bk == 0 && K % p2.bk == 0)) tail = 0;
+    }
     if (tail > 0) {  // whole rounds first, then the narrow remainder as a split contraction
       const int64_t n1 = N - tail;
       const int64_t osz = out_dtype == TF_F32 ? 4 : 2;
       const char* b2 = (const char*)B + (layout_b == TF_OP_KMAJOR ? n1 * ldb : n1) * 2;
       const void* bias2 = bias ? (const char*)bias + n1 * 2 : nullptr;
       const void* mask2 = mask_act ? (const char*)mask_act + n1 * 2 : nullptr;
+      void* so2 = sign_out ? (char*)sign_out + n1 / 8 : nullptr;
+      const void* si2 = sign_in ? (const char*)sign_in + n1 / 8 : nullptr;
       const int rc = gemm_entry(stream, dtype, out_dtype, layout_a, layout_b, M, n1, K, A, lda, B, ldb, C, ldc, 0, 0, bias,
-                                relu, mask_act, ld_mask, workspace, workspace_bytes, nullptr, nullptr, 0, force, alpha);
+                                relu, mask_act, ld_mask, workspace, workspace_bytes, sign_out, sign_in, ld_sign, force, alpha);
       if (rc != TF_OK) return rc;
       return gemm_entry(stream, dtype, out_dtype, layout_a, layout_b, M, tail, K, A, lda, b2, ldb, (char*)C + n1 * osz,
-                        ldc, 0, 0, bias2, relu, mask2, ld_mask, workspace, workspace_bytes, nullptr, nullptr, 0, force,
+                        ldc, 0, 0, bias2, relu, mask2, ld_mask, workspace, workspace_bytes, so2, si2, ld_sign, force,
                         alpha);
     }
   }
