@@ -161,3 +161,23 @@ def test_a_pass_that_raised_leaves_nothing_behind(dev):
     assert not D._pending
     for n in want:
         assert torch.equal(got[n], want[n]), n
+
+
+@pytest.mark.gpu
+def test_forward_on_a_stream_of_its_own(dev):
+    """The engine runs each backward node on the stream of its forward; what the queue launches when the
+    pass ends goes to that stream too, not to the caller's current one."""
+    model, ids = _model(dev)
+    _, want = _step(model, ids)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    model.zero_grad(set_to_none=True)
+    with torch.cuda.stream(side):
+        with torch.autocast("cuda", dtype=torch.float16):
+            _, loss = model(ids, ids)
+        scaled = loss * 1024.0
+    scaled.backward()            # called with the default stream current
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    for n, p in model.named_parameters():
+        assert torch.equal(p.grad, want[n]), n

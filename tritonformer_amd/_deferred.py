@@ -33,6 +33,7 @@ _enabled = False
 _pending = []
 _pending_ln = []
 _task = None
+_stream = None
 _cus = {}
 
 
@@ -146,19 +147,23 @@ def _finish_ln():
 
 
 def _finish():
-    global _task
+    global _task, _stream
     _task = None
     try:
-        _drain(final=True)
-        if _pending_ln:
-            _finish_ln()
+        # on the stream the pass ran on (the engine runs this on the thread that called backward(), whose
+        # current stream is another one when the forward pass ran under a stream of its own)
+        with torch.cuda.stream(_stream):
+            _drain(final=True)
+            if _pending_ln:
+                _finish_ln()
     finally:
+        _stream = None
         _pending.clear()
         _pending_ln.clear()
 
 
 def _join_pass():
-    global _task
+    global _task, _stream
     task = torch._C._current_graph_task_id()
     if task < 0:
         raise RuntimeError("deferred parameter gradients are submitted from inside a backward pass")
@@ -167,6 +172,7 @@ def _join_pass():
         _pending.clear()
         _pending_ln.clear()
         _task = task
+        _stream = torch.cuda.current_stream()
         torch.autograd.Variable._execution_engine.queue_callback(_finish)
 
 
