@@ -84,7 +84,15 @@ def _fill(tiles, cus):
     return tiles / (-(-tiles // cus) * cus)
 
 
-def _pick(items, cus):
+def _fill_split(tiles, cus):
+    """The share of the chip a launch keeps busy when the grouped GEMM may split contractions: at most half
+    a round of tiles runs as cus // tiles slices per tile (fp32 partial sums and a second pass: rated 0.9)."""
+    if 2 * tiles <= cus:
+        return 0.9 * tiles * (cus // tiles) / cus
+    return _fill(tiles, cus)
+
+
+def _pick(items, cus, rate=_fill):
     """Indices of up to _MAX_GROUP products (of the first one's kind) whose tiles best fill whole rounds;
     among equals the oldest, then the most tiles.  Returns (indices, fill)."""
     reach = {0: ()}
@@ -98,7 +106,7 @@ def _pick(items, cus):
     for s, sub in reach.items():
         if not sub:
             continue
-        f = _fill(s, cus)
+        f = rate(s, cus)
         rank = (min(f, _FILL), 0 in sub, s)
         if best_rank is None or rank > best_rank:
             best, best_rank = sub, rank
@@ -118,11 +126,21 @@ def _launch(items):
                     p.grad.add_(g)
 
 
+def _next_launch(items, cus, final):
+    """Indices of the products to launch now, or None to wait for more."""
+    sub, fill = _pick(items, cus)
+    if fill < _FILL:
+        if not final and len(items) < _MAX_PENDING:
+            return None
+        # nothing more is coming (or too much is held): what fills the chip best, split contractions included
+        sub, fill = _pick(items, cus, _fill_split)
+    return sub
+
+
 def _drain(final):
     while _pending:
-        cus = _round(_pending[0].x.device)
-        sub, fill = _pick(_pending, cus)
-        if not final and fill < _FILL and len(_pending) < _MAX_PENDING:
+        sub = _next_launch(_pending, _round(_pending[0].x.device), final)
+        if sub is None:
             return
         items = [_pending[i] for i in sub]
         for i in reversed(sub):
