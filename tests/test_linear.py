@@ -286,9 +286,10 @@ def test_every_tile_configuration_gives_the_same_product(layouts, dev):
 
 @pytest.mark.parametrize("layouts", ["fwd", "dx", "dw"])
 def test_short_contractions_take_every_peeled_form_of_the_main_loop(layouts, dev):
-    """One, two, three, four and five 64-wide stages: the main loop of the direct-to-LDS kernels peels
-    its last two stages (no stage after, one stage after) from the steady state, and its prologue
-    requests the head of the second stage before it waits for the first.  Every tile configuration,
+    """One to nine 64-wide stages: the main loop of the direct-to-LDS kernels peels
+    its last two stages (no stage after, one stage after; three with three LDS buffers) from the steady state, and its
+    prologue requests the head of the second stage (with three buffers: all of it and the head of the third) before it
+    waits for the first.  Every tile configuration,
     against fp32 math, with and without a split that leaves a single stage per slice."""
     from tritonformer_amd import _lib
 
@@ -297,7 +298,7 @@ def test_short_contractions_take_every_peeled_form_of_the_main_loop(layouts, dev
     M, N = 384, 512
     la, lb = {"fwd": (0, 1), "dx": (0, 0), "dw": (1, 1)}[layouts]
     stream = torch.cuda.current_stream().cuda_stream
-    for K in (64, 128, 192, 256, 320):
+    for K in (64, 128, 192, 256, 320, 384, 448, 576):   # (the three-buffer configurations peel three stages and rotate)
         a = torch.randn((M, K) if la == 0 else (K, M), generator=g).half().to(dev)
         b = (torch.randn((N, K) if lb == 0 else (K, N), generator=g) / K ** 0.5).half().to(dev)
         want = (a.float() if la == 0 else a.float().T) @ (b.float().T if lb == 0 else b.float())

@@ -642,8 +642,13 @@ __device__ __forceinline__ void gemm_epilogue_bits(const GemmParams& p, f32x16 (
   }
 }
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR>
+// NS: pipeline stages in LDS.  2: ping-pong -- the loads of a stage are requested while the stage before it is
+// being multiplied, and have one stage's time to arrive.  3: a stage's loads are requested two stages ahead
+// and have two stages' time: for tiles whose stage is short (256x128: half the MFMAs of 256x256 per stage)
+// one stage's time does not cover the latency of operands that come from HBM rather than from the L2.
+template <typename T, int BM, int BN, int BK, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, int NS = 2>
 __device__ __forceinline__ void gemm_dma_body(const GemmParams& p, const int pid) {
+  static_assert(NS == 2 || NS == 3, "two or three pipeline stages");
   constexpr int NW = WM * WN;
   constexpr int WTM = BM / WM, WTN = BN / WN;
   constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -731,7 +736,27 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams& p, const int pid
     PB::advance(pb, p.ldb);
     // the head of step 1 goes out before step 0 is waited for: the two travel together through
     // the cold start instead of one after the other
-    if (nk > 1) {
+    if constexpr (NS == 3) {
+      // three buffers: all of step 1 and the head of step 2
+      if (nk > 1) {
+        PA::issue(pa, smem + STAGE, wave);
+        PB::issue(pb, smem + STAGE + PA::BYTES, wave);
+        PA::advance(pa, p.lda);
+        PB::advance(pb, p.ldb);
+        if (nk > 2) {
+#pragma unroll
+          for (int q = 0; q < NEARLY; ++q) {
+            if (q < PA::PER_WAVE) PA::issue_one(pa, smem + 2 * STAGE, wave, q);
+            else PB::issue_one(pb, smem + 2 * STAGE + PA::BYTES, wave, q - PA::PER_WAVE);
+          }
+          wait_vmcnt<LPS + NEARLY>();  // loads complete in order: all but the youngest LPS + NEARLY = step 0
+        } else {
+          wait_vmcnt<LPS>();
+        }
+      } else {
+        wait_vmcnt<0>();
+      }
+    } else if (nk > 1) {
 #pragma unroll
       for (int q = 0; q < NEARLY; ++q) {
         if (q < PA::PER_WAVE) PA::issue_one(pa, smem + STAGE, wave, q);
@@ -775,23 +800,37 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams& p, const int pid
   };
   // One 64-wide stage.  MORE: another stage follows (hand over to it); MORE2: and one after that
   // (its first loads go out).  Compile-time, so the steady state of the loop has no branch.
-  auto stage = [&](char* cur, char* nxt, auto more_c, auto more2_c) {
-    constexpr bool MORE = decltype(more_c)::value, MORE2 = decltype(more2_c)::value;
+  // With three buffers (NS == 3) everything that is loaded lies one stage further ahead: step 0 sends the
+  // rest of the stage after the next one into the third buffer `far`, the last step the head of the stage
+  // after that into `cur`; MORE3: that stage exists.  The hand-over then waits for all but the youngest
+  // stage's loads.
+  auto stage = [&](char* cur, char* nxt, char* far, auto more_c, auto more2_c, auto more3_c) {
+    constexpr bool MORE = decltype(more_c)::value, MORE2 = decltype(more2_c)::value, MORE3 = decltype(more3_c)::value;
+    constexpr bool LOAD0 = NS == 3 ? MORE2 : MORE;    // step 0 has loads to send (and step 1 pointers to move)
+    constexpr bool LOADL = NS == 3 ? MORE3 : MORE2;   // the last step has
+    char* const dst0 = NS == 3 ? far : nxt;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
       const bool last = ks + 1 == KSTEPS;
       const int first = last ? HAND : 0;                 // first slot that carries work of this step
       const int xfirst = first + RSLOTS < NMFMA ? first + RSLOTS : NMFMA - 1;  // extras: behind the reads
       const int xslots = NMFMA - xfirst;
-      const int nx = !MORE ? 0 : last ? (MORE2 ? NEARLY : 0) : ks == 0 ? LPS - NEARLY : ks == 1 ? LPS : 0;
+      const int nx = last ? (LOADL ? NEARLY : 0) : !LOAD0 ? 0 : ks == 0 ? LPS - NEARLY : ks == 1 ? LPS : 0;
       wait_lgkmcnt<0>();  // the operands of this step were requested a whole step ago
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int m = 0; m < NMFMA; ++m) {
         const int i = m / TN, j = m % TN;
         if (last && m == HAND && MORE) {
-          wait_vmcnt<0>();  // this wave's loads of the next stage have landed
+#ifdef TF_ABL_NO_LOAD_WAIT_TILE
+          if (BM * BN != TF_ABL_NO_LOAD_WAIT_TILE)
+#endif
+#ifndef TF_ABL_NO_LOAD_WAIT
+          wait_vmcnt<(NS == 3 && MORE2) ? LPS : 0>();  // this wave's loads of the next stage have landed
+#endif
+#ifndef TF_ABL_NO_HANDOVER_BARRIER
           barrier();        // ... and everyone's; everyone has read the last operands of `cur`
+#endif
           __builtin_amdgcn_sched_barrier(0);
         }
         acc[i][j] = mfma32(fb[ks & 1][j].template get<v8>(), fa[ks & 1][i].template get<v8>(), acc[i][j]);
@@ -806,8 +845,8 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams& p, const int pid
         if (m >= xfirst) {
 #pragma unroll
           for (int q = (m - xfirst) * nx / xslots; q < (m - xfirst + 1) * nx / xslots; ++q) {
-            if (last) load_item(cur, q);                 // first half of the stage after the next one
-            else if (ks == 0) load_item(nxt, NEARLY + q);  // the rest of the next stage
+            if (last) load_item(cur, q);                 // first half of the stage after the next one (NS == 3: one further)
+            else if (ks == 0) load_item(dst0, NEARLY + q);  // the rest of the next stage (NS == 3: of the one after it)
             else advance_item(q);
           }
         }
@@ -818,12 +857,22 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams& p, const int pid
   typedef std::integral_constant<bool, true> yes_t;
   typedef std::integral_constant<bool, false> no_t;
   int kt = 0;
-  for (; kt + 2 < nk; ++kt) stage(smem + (kt & 1) * STAGE, smem + ((kt + 1) & 1) * STAGE, yes_t(), yes_t());
-  if (kt + 1 < nk) {
-    stage(smem + (kt & 1) * STAGE, smem + ((kt + 1) & 1) * STAGE, yes_t(), no_t());
-    ++kt;
+  if constexpr (NS == 3) {
+    int o0 = 0, o1 = STAGE, o2 = 2 * STAGE;   // buffers of this stage, the next one and the one after it
+    auto rotate = [&]() { const int t = o0; o0 = o1; o1 = o2; o2 = t; ++kt; };
+    for (; kt + 3 < nk; rotate()) stage(smem + o0, smem + o1, smem + o2, yes_t(), yes_t(), yes_t());
+    if (kt + 2 < nk) { stage(smem + o0, smem + o1, smem + o2, yes_t(), yes_t(), no_t()); rotate(); }
+    if (kt + 1 < nk) { stage(smem + o0, smem + o1, smem + o2, yes_t(), no_t(), no_t()); rotate(); }
+    if (kt < nk) stage(smem + o0, smem + o1, smem + o2, no_t(), no_t(), no_t());
+  } else {
+    for (; kt + 2 < nk; ++kt)
+      stage(smem + (kt & 1) * STAGE, smem + ((kt + 1) & 1) * STAGE, nullptr, yes_t(), yes_t(), no_t());
+    if (kt + 1 < nk) {
+      stage(smem + (kt & 1) * STAGE, smem + ((kt + 1) & 1) * STAGE, nullptr, yes_t(), no_t(), no_t());
+      ++kt;
+    }
+    if (kt < nk) stage(smem + (kt & 1) * STAGE, smem + ((kt + 1) & 1) * STAGE, nullptr, no_t(), no_t(), no_t());
   }
-  if (kt < nk) stage(smem + (kt & 1) * STAGE, smem + ((kt + 1) & 1) * STAGE, no_t(), no_t());
 
   static_assert(NW * 32 * (WTN * 4 + 16) <= 2 * STAGE, "epilogue staging must fit in the pipeline LDS");
   static_assert(NW * 32 * (WTN * 2 + 16) + BM * BN / 8 <= 2 * STAGE, "... and so must the image of a tile's sign bits behind it");
@@ -854,12 +903,8 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams& p, const int pid
     } else {
       // the two sign-bit launches of a fused MLP, on full tiles of a plain (unchunked) result whose bit rows take
       // 16-byte pieces: write-outs of their own, nothing tested per store
-#ifdef TF_NO_FAST_BITS
-      const bool bits_fast = false &&
-#else
-      const bool bits_fast = full &&
-#endif !p.mask && !p.alpha && p.chunk_skip == 0 && p.ldsign % 16 == 0 &&
-                             (reinterpret_cast<uintptr_t>(p.sign_out) & 15) == 0;
+      const bool bits_fast = full && !p.mask && !p.alpha && p.chunk_skip == 0 && p.ldsign % 16 == 0 &&
+                             ((reinterpret_cast<uintptr_t>(p.sign_out) | reinterpret_cast<uintptr_t>(p.sign_in)) & 15) == 0;
       if (plain && full) gemm_epilogue_lds<T, T, TM, TN, WTM, WTN, true, true>(p, acc, smem, m0, n0, wm, wn, wave, lane);
       else if (plain) gemm_epilogue_lds<T, T, TM, TN, WTM, WTN, true>(p, acc, smem, m0, n0, wm, wn, wave, lane);
       else if (bits_fast && p.sign_out && p.relu) gemm_epilogue_bits<T, BM, BN, TM, TN, WTM, WTN, true>(p, acc, smem, m0, n0, wm, wn, wave, lane, sign_bytes);
@@ -869,10 +914,10 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams& p, const int pid
   }
 }
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, int WPE, bool A_KMAJOR, bool B_KMAJOR>
+template <typename T, int BM, int BN, int BK, int WM, int WN, int WPE, bool A_KMAJOR, bool B_KMAJOR, int NS = 2>
 __global__ __launch_bounds__(WM* WN * 64, WPE) void gemm_dma_kernel(GemmParams p) {
   const int pid = (p.flags & 1) ? (int)blockIdx.x : remap_xcd(blockIdx.x, p.tiles_m * p.tiles_n * p.splits, p.xcds);
-  gemm_dma_body<T, BM, BN, BK, WM, WN, A_KMAJOR, B_KMAJOR>(p, pid);
+  gemm_dma_body<T, BM, BN, BK, WM, WN, A_KMAJOR, B_KMAJOR, NS>(p, pid);
 }
 
 // Up to eight independent products of one operand layout in ONE launch: workgroup ids
@@ -990,8 +1035,8 @@ static const TileCfg kCfgs[] = {
     {128, 128, 64, 4, 0},  // 1: register-staged, wave tile 64x64, any shape / alignment
     {256, 256, 64, 8, 1},  // 2: direct-to-LDS, 128 KB LDS, one workgroup per CU, wave tile 128x64
     {128, 128, 64, 4, 1},  // 3: direct-to-LDS, 64 KB LDS, two workgroups per CU, wave tile 64x64
-    {256, 128, 64, 8, 1},  // 4: direct-to-LDS, 96 KB LDS, waves 4x2, wave tile 64x64
-    {128, 256, 64, 8, 1},  // 5: direct-to-LDS, 96 KB LDS, waves 2x4, wave tile 64x64
+    {256, 128, 64, 8, 1},  // 4: direct-to-LDS, three stages = 144 KB LDS, waves 4x2, wave tile 64x64
+    {128, 256, 64, 8, 1},  // 5: direct-to-LDS, three stages = 144 KB LDS, waves 2x4, wave tile 64x64
 };
 constexpr int kNumCfgs = (int)(sizeof(kCfgs) / sizeof(kCfgs[0]));
 
@@ -1040,7 +1085,10 @@ static GemmPlan plan_for(int cfg, int64_t M, int64_t N, int64_t K, double* cost_
   if (pl.splits < 1) pl.splits = 1;
   if (cost_us) {
     const double fixed = pl.bm * pl.bn >= 256 * 256 ? 10.0 : 7.0;
-    const double per_step = pl.bm * pl.bn >= 256 * 256 ? 1.65 : (pl.bm * pl.bn >= 256 * 128 ? 1.15 : 1.1);
+#ifndef TF_STEP_256x128
+#define TF_STEP_256x128 1.0
+#endif
+    const double per_step = pl.bm * pl.bn >= 256 * 256 ? 1.65 : (pl.bm * pl.bn >= 256 * 128 ? TF_STEP_256x128 : 1.1);
     const int64_t rounds = (tiles * pl.splits + slots - 1) / slots;
     double c = (double)rounds * (fixed + per_step * (double)steps_per);
     if (pl.splits > 1) c += 3.0 + (pl.splits + 0.5) * (double)M * (double)N * 4.0 / 5.0e6;
@@ -1099,11 +1147,11 @@ static int launch_one(hipStream_t st, const GemmParams& p) {
   return TF_OK;
 }
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, int WPE, bool AK, bool BKM>
+template <typename T, int BM, int BN, int BK, int WM, int WN, int WPE, bool AK, bool BKM, int NS = 2>
 static int launch_dma(hipStream_t st, const GemmParams& p) {
-  constexpr int lds = 2 * (BM + BN) * BK * 2;
+  constexpr int lds = NS * (BM + BN) * BK * 2;
   static_assert(lds <= 160 * 1024, "LDS budget");
-  auto kernel = gemm_dma_kernel<T, BM, BN, BK, WM, WN, WPE, AK, BKM>;
+  auto kernel = gemm_dma_kernel<T, BM, BN, BK, WM, WN, WPE, AK, BKM, NS>;
   static bool once = (allow_big_lds(kernel, lds), true);
   (void)once;
   const unsigned grid = (unsigned)(p.tiles_m * p.tiles_n * p.splits);
@@ -1116,14 +1164,20 @@ static int launch_dma(hipStream_t st, const GemmParams& p) {
 // The register-staged kernel handles everything (ragged extents, unaligned
 // pointers); the direct-to-LDS kernel needs the vector conditions and a
 // contraction extent that is a multiple of its BK.
+// LDS stages of the 256x128 / 128x256 configurations (a diagnostic build may impose 2)
+#ifndef TF_STAGES_NARROW
+#define TF_STAGES_NARROW 3
+#endif
+constexpr int kStagesNarrow = TF_STAGES_NARROW;
+
 template <typename T, bool AK, bool BKM, bool VEC>
 static int launch_cfg(hipStream_t st, const GemmPlan& pl, const GemmParams& p) {
   if (kCfgs[pl.cfg].dma && VEC && p.K % pl.bk == 0) {
     switch (pl.cfg) {
       case 2: return launch_dma<T, 256, 256, 64, 2, 4, 2, AK, BKM>(st, p);
       case 3: return launch_dma<T, 128, 128, 64, 2, 2, 2, AK, BKM>(st, p);
-      case 4: return launch_dma<T, 256, 128, 64, 4, 2, 2, AK, BKM>(st, p);
-      case 5: return launch_dma<T, 128, 256, 64, 2, 4, 2, AK, BKM>(st, p);
+      case 4: return launch_dma<T, 256, 128, 64, 4, 2, 2, AK, BKM, kStagesNarrow>(st, p);
+      case 5: return launch_dma<T, 128, 256, 64, 2, 4, 2, AK, BKM, kStagesNarrow>(st, p);
     }
   }
   if (pl.bm == 256 && pl.bn == 256) return launch_one<T, 256, 256, 64, 2, 4, AK, BKM, VEC>(st, p);
