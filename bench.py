@@ -42,7 +42,7 @@ PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per GEMM launch at the headline workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # scaled against a streaming kernel of known size (profiles/hbm_traffic_410m_step.md)
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = {"gpt2-410m-ctx2048-bs4": 158.7e6}
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = {"gpt2-410m-ctx2048-bs4": 170.5e6}
 
 WORKLOADS = {
     # name: (layers, d, heads, head_dim, ffn, seq, batch, linear_bias, alibi)

@@ -547,3 +547,42 @@ def test_gemm_scaled_is_alpha_times_the_product(case, dtype, dev):
         out = torch.full((M, N), float("nan"), dtype=out_dtype, device=dev)
         K_mod.gemm_scaled(a, la, M, K, a.stride(0), b, lb, N, b.stride(0), alpha, out)
         assert torch.equal(out, (plain * alpha).to(out_dtype)), (case, out_dtype)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("pitch,shift", [(40, 0), (48, 8), (37, 0)])
+def test_sign_bit_rows_of_any_pitch_and_alignment(pitch, shift, dev):
+    """tf_gemm_relu_bits through the C ABI with bit rows that the 16-byte write-out cannot take (a pitch that
+    is no multiple of 16 bytes, a buffer that starts 8 bytes into a 16-byte line): the byte-wise write-out
+    serves them -- same activation, same bits, and the masked product read back from those rows equals the
+    one that reads the activation (kernels/activation.py:27-44)."""
+    import numpy as np
+    from tritonformer_amd import _lib
+    from tritonformer_amd import kernels as K
+
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(41)
+    m, d, f = 512, 256, 256
+    x = torch.randn(m, d, generator=g).half().to(dev)
+    w1 = (torch.randn(d, f, generator=g) / d ** 0.5).half().to(dev)
+    w2 = (torch.randn(f, d, generator=g) / f ** 0.5).half().to(dev)
+    dy = torch.randn(m, d, generator=g).half().to(dev)
+    hidden = torch.empty(m, f, dtype=torch.float16, device=dev)
+    raw = torch.zeros(m * pitch + 64, dtype=torch.uint8, device=dev)
+    bits = raw[shift:shift + m * pitch].view(m, pitch)
+    st = _lib.stream_ptr()
+    # forward: x (m, d) k-contiguous, W1 (d, f) k-strided
+    rc = lib.tf_gemm_relu_bits(st, 0, 0, 0, 1, m, f, d, x.data_ptr(), d, w1.data_ptr(), f, hidden.data_ptr(), f, None,
+                               bits.data_ptr(), None, pitch)
+    assert rc == 0
+    want_h = K.gemm(x.view(1, m, d), w1, None, True).view(m, f)
+    assert torch.equal(hidden, want_h)
+    expect = np.packbits((want_h > 0).cpu().numpy(), axis=1, bitorder="little")
+    assert np.array_equal(bits[:, : f // 8].cpu().numpy(), expect)
+    assert not bits[:, f // 8:].any()                      # nothing written between the rows
+    # backward: dH = (dY W2^T) masked by the bits; W2 (f, d) read with the contraction contiguous
+    dh = torch.empty(m, f, dtype=torch.float16, device=dev)
+    rc = lib.tf_gemm_relu_bits(st, 0, 0, 0, 0, m, f, d, dy.data_ptr(), d, w2.data_ptr(), d, dh.data_ptr(), f, None,
+                               None, bits.data_ptr(), pitch)
+    assert rc == 0
+    assert torch.equal(dh, K.mm(dy.view(1, m, d), w2.T, mask_act=want_h.view(1, m, f)).view(m, f))
