@@ -828,9 +828,10 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams& p, const int pid
 #ifndef TF_ABL_NO_LOAD_WAIT
           wait_vmcnt<(NS == 3 && MORE2) ? LPS : 0>();  // this wave's loads of the next stage have landed
 #endif
-#ifndef TF_ABL_NO_HANDOVER_BARRIER
-          barrier();        // ... and everyone's; everyone has read the last operands of `cur`
+#ifdef TF_ABL_NO_HANDOVER_BARRIER_TILE
+          if (BM * BN != TF_ABL_NO_HANDOVER_BARRIER_TILE)
 #endif
+          barrier();        // ... and everyone's; everyone has read the last operands of `cur`
           __builtin_amdgcn_sched_barrier(0);
         }
         acc[i][j] = mfma32(fb[ks & 1][j].template get<v8>(), fa[ks & 1][i].template get<v8>(), acc[i][j]);
