@@ -822,12 +822,13 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams& p, const int pid
       for (int m = 0; m < NMFMA; ++m) {
         const int i = m / TN, j = m % TN;
         if (last && m == HAND && MORE) {
+          // (Measurement switches, never defined by the build: TF_ABL_NO_LOAD_WAIT_TILE / TF_ABL_NO_HANDOVER_BARRIER_TILE
+          // = BM * BN of the configuration whose wait / barrier is compiled out.  The results of such a build are
+          // wrong; its step time says what the wait costs -- how the need for a third stage was found.)
 #ifdef TF_ABL_NO_LOAD_WAIT_TILE
           if (BM * BN != TF_ABL_NO_LOAD_WAIT_TILE)
 #endif
-#ifndef TF_ABL_NO_LOAD_WAIT
           wait_vmcnt<(NS == 3 && MORE2) ? LPS : 0>();  // this wave's loads of the next stage have landed
-#endif
 #ifdef TF_ABL_NO_HANDOVER_BARRIER_TILE
           if (BM * BN != TF_ABL_NO_HANDOVER_BARRIER_TILE)
 #endif
