@@ -1071,12 +1071,37 @@ static GemmPlan plan_for(int cfg, int64_t M, int64_t N, int64_t K, double* cost_
   // gradients: few output tiles, long contraction); never beyond one full round of
   // workgroups, and every slice keeps at least 16 steps so that the fp32 partial
   // traffic stays small.
+#ifndef TF_STEP_256x128
+#define TF_STEP_256x128 1.0
+#endif
+  const double fixed = pl.bm * pl.bn >= 256 * 256 ? 10.0 : 7.0;
+  const double per_step = pl.bm * pl.bn >= 256 * 256 ? 1.65 : (pl.bm * pl.bn >= 256 * 128 ? TF_STEP_256x128 : 1.1);
+  auto cost_of = [&](int64_t nsplit, int64_t steps) {
+    const int64_t rounds = (tiles * nsplit + slots - 1) / slots;
+    double c = (double)rounds * (fixed + per_step * (double)steps);
+    if (nsplit > 1) c += 3.0 + (nsplit + 0.5) * (double)M * (double)N * 4.0 / 5.0e6;
+    return c;
+  };
   int64_t splits = 1;
   if (tiles <= slots / 2) {
     splits = slots / tiles;
     const int64_t max_by_k = ksteps / 16 > 0 ? ksteps / 16 : 1;
     if (splits > max_by_k) splits = max_by_k;
     if (splits > 16) splits = 16;
+  }
+  // A long contraction whose tiles leave part of a round idle (0.75 of a round: the LM-head input gradient
+  // of a narrow model) may be cheaper in more, shorter slices that fill whole rounds: by the cost model,
+  // among slice counts that keep 16 steps per slice, and only when it wins by a tenth.
+#ifdef TF_NO_SPLIT_SEARCH
+  if (false) {
+#else
+  if (allow_split && force_splits <= 0 && tiles % slots != 0 && ksteps >= 256) {
+#endif
+    double best = cost_of(splits, (ksteps + splits - 1) / splits) * 0.9;
+    for (int64_t sp = 2; sp <= 16 && ksteps / sp >= 16; ++sp) {
+      const double c = cost_of(sp, (ksteps + sp - 1) / sp);
+      if (c < best) { best = c; splits = sp; }
+    }
   }
   if (force_splits > 0) splits = force_splits;
   if (!allow_split) splits = 1;
@@ -1085,17 +1110,7 @@ static GemmPlan plan_for(int cfg, int64_t M, int64_t N, int64_t K, double* cost_
   pl.k_per_split = (int)(steps_per * pl.bk);
   pl.splits = (int)((ksteps + steps_per - 1) / steps_per);
   if (pl.splits < 1) pl.splits = 1;
-  if (cost_us) {
-    const double fixed = pl.bm * pl.bn >= 256 * 256 ? 10.0 : 7.0;
-#ifndef TF_STEP_256x128
-#define TF_STEP_256x128 1.0
-#endif
-    const double per_step = pl.bm * pl.bn >= 256 * 256 ? 1.65 : (pl.bm * pl.bn >= 256 * 128 ? TF_STEP_256x128 : 1.1);
-    const int64_t rounds = (tiles * pl.splits + slots - 1) / slots;
-    double c = (double)rounds * (fixed + per_step * (double)steps_per);
-    if (pl.splits > 1) c += 3.0 + (pl.splits + 0.5) * (double)M * (double)N * 4.0 / 5.0e6;
-    *cost_us = c;
-  }
+  if (cost_us) *cost_us = cost_of(pl.splits, steps_per);
   return pl;
 }
 
