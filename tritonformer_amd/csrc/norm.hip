@@ -158,17 +158,35 @@ __global__ __launch_bounds__(256) void ln_bwd_vec(int64_t rows, int d, const T* 
                                                    const TP* __restrict__ gamma, const float* __restrict__ mean,
                                                    const float* __restrict__ rstd, T* __restrict__ dx,
                                                    int64_t lddx, float* __restrict__ partial) {
-  extern __shared__ float red[];  // [4][d]
+  extern __shared__ float red[];  // [4][d], and behind it [d] for gamma when G_LDS
+  // Wide rows (NV >= 4) keep gamma in LDS as fp32 and read a chunk where it is used: held in registers its
+  // 8 * NV values pushed the kernel past 256 registers, one wave per SIMD and one workgroup per CU, so that
+  // the 512 workgroups of a launch ran in two turns (d = 2048: 23.4 us per launch with it, 67 MB).
+  constexpr bool G_LDS = NV >= 4;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int nchunk = d >> 3;
-  float g[NV][8], dg[NV][8], db[NV][8];
+  float* const gam = red + 4 * d;
+  float g[G_LDS ? 1 : NV][8], dg[NV][8], db[NV][8];
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
     const int c = lane + i * 64;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) { dg[i][e] = 0.f; db[i][e] = 0.f; g[i][e] = 0.f; }
-    if (c < nchunk) load8<TP>(gamma + c * 8, g[i]);
+    for (int e = 0; e < 8; ++e) { dg[i][e] = 0.f; db[i][e] = 0.f; }
+    if constexpr (!G_LDS) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) g[i][e] = 0.f;
+      if (c < nchunk) load8<TP>(gamma + c * 8, g[i]);
+    }
+  }
+  if constexpr (G_LDS) {
+    for (int c = threadIdx.x; c < nchunk; c += 256) {
+      float gv[8];
+      load8<TP>(gamma + c * 8, gv);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) gam[c * 8 + e] = gv[e];
+    }
+    __syncthreads();
   }
   const float inv_d = 1.0f / (float)d;
   const int64_t stride = (int64_t)gridDim.x * kRowsPerBlock;
@@ -197,14 +215,16 @@ __global__ __launch_bounds__(256) void ln_bwd_vec(int64_t rows, int d, const T* 
     for (int i = 0; i < NV; ++i) {
       const int c = lane + i * 64;
       if (c < nchunk) {
-        float xv[8], dv[8];
+        float xv[8], dv[8], gl[8];
         unpack8<T>(raw_x[i], xv);
         unpack8<T>(raw_dy[i], dv);
         if (ADD) unpack8<T>(raw_ds[i], ds[i]);
 #pragma unroll
+        for (int e = 0; e < 8; ++e) gl[e] = G_LDS ? gam[c * 8 + e] : g[G_LDS ? 0 : i][e];
+#pragma unroll
         for (int e = 0; e < 8; ++e) {
           xh[i][e] = (xv[e] - mu) * rs;
-          gd[i][e] = dv[e] * g[i][e];
+          gd[i][e] = dv[e] * gl[e];
           s1 += gd[i][e] * xh[i][e];
           s2 += gd[i][e];
           dg[i][e] += dv[e] * xh[i][e];
@@ -657,7 +677,7 @@ static int ln_bwd_launch(hipStream_t st, int64_t rows, int64_t d, const void* dy
              aligned16(gamma);
   if (ADD) vec = vec && row_vectorizable<T>(dsum, d, lddsum);
   const int nv = vec ? pick_nv(d / 8) : 0;
-  const size_t lds = (size_t)4 * d * sizeof(float);
+  const size_t lds = (size_t)(nv >= 4 ? 5 : 4) * d * sizeof(float);  // wide rows keep gamma there too
 #define LN_BWD(NV)                                                                                                \
   ln_bwd_vec<T, TP, NV, ADD><<<dim3(parts), dim3(256), lds, st>>>(rows, (int)d, (const T*)dy, lddy, (const T*)dsum,   \
                                                                   lddsum, (const T*)x, ldx, (const TP*)gamma, mean, \
