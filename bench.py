@@ -547,6 +547,8 @@ def main():
                    "seq_len": S, "global_batch": B, "vocab": VOCAB, "linear_bias": lin_bias, "alibi": alibi,
                    "master_weights": "fp32", "autocast": args.dtype, "parallelism": "single GPU",
                    "protocol": "reference README.md:62-77: forward under autocast, loss.backward() unscaled, no optimizer",
+                   "weight_gradients": "launched by the model's gradient queue in whole rounds of workgroups, in param.grad "
+                                       "when backward() returns (`weight_gradients_in_layer` has the in-layer launches)",
                    "weight_casts": "every forward pass" if args.recast else
                                    "16-bit copies of the unchanged fp32 weights kept between steps (keyed on the "
                                    "parameters' version counters); `recast_each_step` has the other mode"},
