@@ -152,6 +152,8 @@ FAMILY_ENTRY_POINTS = {
     "tf_layernorm_bwd": ("layernorm", lambda a: 6.0 * a[3] * a[4]),
     "tf_add_layernorm_fwd": ("layernorm", lambda a: 8.0 * a[3] * a[4]),
     "tf_add_layernorm_bwd": ("layernorm", lambda a: 8.0 * a[3] * a[4]),
+    # second stage of all LayerNorms of a pass at once: 512 partial rows (row passes over >= 2048 rows) of 2d fp32 each
+    "tf_layernorm_param_grads": ("layernorm", lambda a: 512.0 * 2 * a[2] * 4 * a[3]),
     "tf_cross_entropy_fwd": ("cross_entropy", lambda a: 2.0 * a[2] * a[3]),
     "tf_cross_entropy_fwd_grad": ("cross_entropy", lambda a: 4.0 * a[2] * a[3]),
     "tf_cross_entropy_bwd": ("cross_entropy", lambda a: 4.0 * a[2] * a[3]),
