@@ -143,7 +143,7 @@ int tf_gemm_scaled(void* stream, int dtype, int out_dtype, int layout_a, int lay
                    void* C, int64_t ldc, const float* alpha,
                    void* workspace, int64_t workspace_bytes);
 
-/* `count` (1..8) independent products of one dtype and one pair of operand layouts,
+/* `count` (1..16) independent products of one dtype and one pair of operand layouts,
  * no bias / ReLU / mask, each with the arguments of tf_gemm_out_chunked.  When every
  * problem meets the fast-path preconditions and both operands are TF_OP_KMINOR (the
  * weight-gradient form x^T . dy of tritonformer/linear.py:24-25), all of them run in

@@ -131,7 +131,7 @@ def test_gemm_rejects_bad_arguments():
     assert lib.tf_gemm_group_workspace_bytes(1, 1, 2, probs) == 2 * 2 * 1024 * 4096 * 4
     assert lib.tf_gemm_workspace_bytes(1, 1, 1024, 4096, 8192) == 4 * 1024 * 4096 * 4
     assert lib.tf_gemm_group(None, 0, 2, 1, 1, 2, probs, None, 0) == -5
-    assert lib.tf_gemm_group(None, 0, 2, 1, 1, 9, probs, FAKE, 1 << 40) == -1
+    assert lib.tf_gemm_group(None, 0, 2, 1, 1, 17, probs, FAKE, 1 << 40) == -1
     assert lib.tf_gemm_group(None, 2, 2, 1, 1, 2, probs, FAKE, 1 << 40) == -2
     assert lib.tf_gemm_group(None, 0, 1, 1, 1, 2, probs, FAKE, 1 << 40) == -2
     ptrs = (ctypes.c_void_p * 3)(FAKE, FAKE, FAKE)

@@ -183,3 +183,32 @@ def test_forward_on_a_stream_of_its_own(dev):
     torch.cuda.synchronize()
     for n, p in model.named_parameters():
         assert torch.equal(p.grad, want[n]), n
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fuse_qkv", [False, True])
+def test_reference_named_linears_defer_too(fuse_qkv, dev):
+    """With the model-level fusions off the model is the reference's graph node for node
+    (LinearNoBias x 4 + LinearNoBiasReLU / LinearNoBias per block, transformer.py:153-217, the LM head a
+    Linear as well): their weight gradients take the queue too, and equal the in-layer ones; with
+    FUSE_QKV alone the packed projection hands over one product for three weights."""
+    model, ids = _model(dev)
+    flags = ("FUSE_QKV", "FUSE_MLP", "FUSE_ATTN_BLOCK", "FUSE_ADD_LN", "FUSE_EMBED", "FUSE_HEAD")
+    saved = {n: getattr(TM, n) for n in flags}
+    try:
+        for n in flags:
+            setattr(TM, n, False)
+        TM.FUSE_QKV = fuse_qkv
+        TM.DEFER_DW = False
+        loss0, g0 = _step(model, ids)
+        TM.DEFER_DW = True
+        loss1, g1 = _step(model, ids)
+        _, g2 = _step(model, ids)
+    finally:
+        TM.DEFER_DW = True
+        for n, v in saved.items():
+            setattr(TM, n, v)
+    assert loss0 == loss1 and not D._pending and not D._pending_ln
+    for n in g0:
+        assert g1[n].dtype == g0[n].dtype and rel_l2(g1[n], g0[n]) < 1e-5, n
+        assert torch.equal(g1[n], g2[n]), n

@@ -448,7 +448,7 @@ def test_grouped_weight_gradients_equal_separate_products(case, dev):
             again = K.mm_dw_group(pairs, out_dtype=od, chunks=chunks)   # fixed summation order: the same bits
             assert all(torch.equal(a, b) for a, b in zip(again, outs))
     with pytest.raises(ValueError):
-        K.mm_dw_group(pairs * 9)
+        K.mm_dw_group(pairs * 17)
 
 
 @pytest.mark.gpu

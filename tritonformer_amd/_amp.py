@@ -86,6 +86,9 @@ def amp_fwd(fwd=None, *, keep=()):
         # dtypes the caller passed in, before any autocast cast (fp32 master weights)
         ctx.arg_dtypes = tuple(a.dtype if isinstance(a, torch.Tensor) else None for a in args)
         ctx.amp_active = torch.is_autocast_enabled("cuda")  # for bodies that cast their `keep` arguments themselves
+        # the parameters as the caller holds them (autocast hands the body 16-bit copies): where a deferred
+        # gradient is delivered
+        ctx.arg_params = tuple(a if isinstance(a, torch.nn.Parameter) else None for a in args)
         if ctx.amp_active:
             dtype = torch.bfloat16 if ctx._dtype == torch.bfloat16 else torch.float16
             with torch.autocast(device_type="cuda", enabled=False):

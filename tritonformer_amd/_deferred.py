@@ -3,8 +3,8 @@
 A weight gradient dW = X^T dY is needed by nobody until the backward pass ends, and the output of one
 such product has few 256x256 tiles (16 to 64 per weight of the 410M model on 256 CUs): launched where
 the reference launches it (linear.py:21-25, inside the layer's backward) it fills the chip only by
-splitting its contraction, which costs fp32 partial sums and a second pass.  Here the block Functions
-hand their (X, dY) pairs over instead; products of several layers are launched together as soon as their
+splitting its contraction, which costs fp32 partial sums and a second pass.  Here the linear and block
+Functions that run inside the model's forward hand their (X, dY) pairs over instead; products of several layers are launched together as soon as their
 tiles make (nearly) whole rounds of one workgroup per CU, unsplit, and what is left goes when the
 engine finishes the pass.  The gradients are complete, on the stream the pass ran on, when
 ``loss.backward()`` returns -- the same contract as before -- but they reach ``param.grad`` directly
@@ -22,12 +22,12 @@ import torch
 
 from .kernels import layernorm_param_grads, mm_dw_group
 
-# products per launch (the grouped GEMM entry point takes up to eight)
-_MAX_GROUP = 8
+# products per launch (the grouped GEMM entry point takes up to sixteen)
+_MAX_GROUP = 16
 # a launch goes as soon as its tiles fill this share of a whole number of rounds
 _FILL = 0.97
 # pending products beyond which the oldest are launched whatever they fill (bounds the memory held)
-_MAX_PENDING = 12
+_MAX_PENDING = 24
 
 _enabled = False
 _pending = []

@@ -922,15 +922,16 @@ __global__ __launch_bounds__(WM* WN * 64, WPE) void gemm_dma_kernel(GemmParams p
   gemm_dma_body<T, BM, BN, BK, WM, WN, A_KMAJOR, B_KMAJOR, NS>(p, pid);
 }
 
-// Up to eight independent products of one operand layout in ONE launch: workgroup ids
+// Up to sixteen independent products of one operand layout in ONE launch: workgroup ids
 // [first[i], first[i+1]) belong to problem i.  Used for weight gradients, whose output has
 // few tiles: side by side they fill the chip with fewer, longer contraction slices.
-constexpr int kMaxGroup = 8;
+constexpr int kMaxGroup = 16;
 struct GemmGroup {
   GemmParams p[kMaxGroup];
   int first[kMaxGroup + 1];
   int count;
 };
+static_assert(sizeof(GemmGroup) <= 4000, "the group travels as a kernel argument (4 KB of them at most)");
 template <typename T, int BM, int BN, int BK, int WM, int WN, int WPE, bool A_KMAJOR, bool B_KMAJOR>
 __global__ __launch_bounds__(WM* WN * 64, WPE) void gemm_dma_group_kernel(GemmGroup g) {
   // (a group with a split tail keeps the ids as dealt, round-robin over the XCDs: whole tiles first, on every

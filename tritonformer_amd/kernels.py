@@ -204,13 +204,13 @@ def mm_dw(x, grad, out_dtype=None, chunks=1):
 
 
 def mm_dw_group(pairs, out_dtype=None, chunks=None):
-    """``[mm_dw(x, g) for x, g in pairs]`` (up to eight weight gradients that are available
+    """``[mm_dw(x, g) for x, g in pairs]`` (up to sixteen weight gradients that are available
     at the same time) through ONE launch where the kernel's preconditions allow: products
     whose outputs have few tiles then share the GPU instead of each splitting its contraction
     into many slices.  ``chunks[i] > 1`` as in mm_dw."""
     chunks = list(chunks) if chunks is not None else [1] * len(pairs)
-    if not 1 <= len(pairs) <= 8 or len(chunks) != len(pairs):
-        raise ValueError("mm_dw_group takes 1..8 (x, grad) pairs")
+    if not 1 <= len(pairs) <= 16 or len(chunks) != len(pairs):
+        raise ValueError("mm_dw_group takes 1..16 (x, grad) pairs")
     probs = (_lib.GemmProblem * len(pairs))()
     outs, keep = [], []
     dt = pairs[0][0].dtype

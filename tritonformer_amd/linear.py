@@ -23,6 +23,13 @@ def _bias_grad(ctx, grad, index):
     return unbroadcast_leading(grad, torch.float32 if ctx.arg_dtypes[index] == torch.float32 else None)
 
 
+def _deferral_target(ctx, index=1):
+    """The weight parameter passed at ``index`` when its gradient is to go through the model's queue
+    (several layers' weight gradients in one launch), else None: call in forward, keep on ctx."""
+    w = ctx.arg_params[index]
+    return w if w is not None and _deferred.active() and GROUP_DW and _deferred.deferrable((w,)) else None
+
+
 def _grads(ctx, grad_output, inputs, weights):
     """dX = dY W^T (W read as stored, contraction along its rows) and
     dW = X^T dY with the batch folded into the contraction
@@ -32,7 +39,11 @@ def _grads(ctx, grad_output, inputs, weights):
         # an fp32 master weight (cast to 16 bit by autocast on the way in) gets its
         # gradient straight from the fp32 accumulators instead of a rounded copy
         master = torch.float32 if ctx.arg_dtypes[1] == torch.float32 else None
-        grad_weights = mm_dw(inputs, grad_output, out_dtype=master)
+        if getattr(ctx, "defer_to", None) is not None:
+            # launched later, together with those of other layers, in whole rounds of workgroups
+            _deferred.submit([(inputs, grad_output, 1, (ctx.defer_to,), master)])
+        else:
+            grad_weights = mm_dw(inputs, grad_output, out_dtype=master)
     # the input gradient last: it is what the next kernel of the backward pass reads
     grad_input = mm(grad_output, weights.T) if ctx.needs_input_grad[0] else None
     return grad_input, grad_weights
@@ -45,6 +56,7 @@ class LinearNoBias(Function):
     @amp_fwd
     def forward(ctx, input, weight):
         ctx.save_for_backward(input, weight)
+        ctx.defer_to = _deferral_target(ctx)
         return mm(input, weight)
 
     @staticmethod
@@ -61,6 +73,7 @@ class LinearBias(Function):
     @amp_fwd
     def forward(ctx, input, weight, bias):
         ctx.save_for_backward(input, weight)
+        ctx.defer_to = _deferral_target(ctx)
         return gemm(input, weight, bias, False)
 
     @staticmethod
@@ -80,6 +93,7 @@ class LinearNoBiasReLU(Function):
     def forward(ctx, input, weight):
         out_w_act = mm(input, weight, True)
         ctx.save_for_backward(input, weight, out_w_act)
+        ctx.defer_to = _deferral_target(ctx)
         return out_w_act
 
     @staticmethod
@@ -98,6 +112,7 @@ class LinearBiasReLU(Function):
     def forward(ctx, input, weight, bias):
         out_w_act = gemm(input, weight, bias, True)
         ctx.save_for_backward(input, weight, out_w_act)
+        ctx.defer_to = _deferral_target(ctx)
         return out_w_act
 
     @staticmethod
@@ -192,12 +207,17 @@ class PackedLinearNoBias(Function):
         ctx.save_for_backward(input, packed)
         ctx.count = len(weights)
         ctx.weight_dtype = weights[0].dtype
+        ctx.defer_to = weights if _deferred.active() and GROUP_DW and _deferred.deferrable(weights) else None
         return mm(input, packed)
 
     @staticmethod
     @amp_bwd
     def backward(ctx, grad_output):
         input, packed = ctx.saved_tensors
+        if ctx.defer_to is not None:
+            _deferred.submit([(input, grad_output, ctx.count, ctx.defer_to, ctx.weight_dtype)])
+            grad_input = mm(grad_output, packed.T) if ctx.needs_input_grad[0] else None
+            return (grad_input,) + (None,) * ctx.count
         grad_w = mm_dw(input, grad_output, out_dtype=ctx.weight_dtype, chunks=ctx.count)
         grad_input = mm(grad_output, packed.T) if ctx.needs_input_grad[0] else None
         return (grad_input,) + tuple(grad_w[j] for j in range(ctx.count))
